@@ -1,0 +1,129 @@
+"""The cache on the GPU: paged keys and values for groups of layers, fixed-size state for each
+sequence, and the ledger that says who holds what.
+
+Cache entries (one per layer that keeps keys and values, as the model's schedule numbers them)
+with the same :class:`KVSpec` form a *group* with storage of its own:
+    keys    [entries, blocks, kv_heads, 64, head_dim]
+    values  [entries, blocks, kv_heads, 16, head_dim, 4]      (four positions interleaved)
+All groups share one block table per sequence, because a sequence is equally long in all of
+them.  Fixed-size state ([entries, slots, *shape], zeroed when a slot is handed out) lives beside
+it for mixers that carry state instead of, or in addition to, keys and values.
+"""
+
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from ..kernels import library as K
+from .ledger import BLOCK, CacheLedger
+
+
+@dataclass(frozen=True)
+class KVSpec:
+    """What a mixer keeps per token: heads and head size; ``window`` > 0 means that only the last
+    ``window`` positions are ever read."""
+    kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """What a mixer keeps per sequence, independent of its length."""
+    shape: Tuple[int, ...]
+    dtype: str = "float32"
+
+
+class KVGroup:
+    def __init__(self, spec, entries, n_blocks, dtype, device):
+        self.spec, self.entries, self.n_blocks = spec, entries, n_blocks
+        shape = (entries, n_blocks, spec.kv_heads, BLOCK, spec.head_dim)
+        self.keys = torch.zeros(shape, dtype=dtype, device=device)
+        self.values = torch.zeros(shape, dtype=dtype, device=device)
+
+    def view(self, entry, block_table, max_blocks):
+        """The kernels' view of one entry with the step's block table [n_seqs, max_blocks]."""
+        return K.KvView(keys=self.keys[entry].data_ptr(), values=self.values[entry].data_ptr(),
+                        blocks=block_table.data_ptr(), max_blocks=max_blocks,
+                        kv_heads=self.spec.kv_heads, head_dim=self.spec.head_dim)
+
+
+class StateGroup:
+    def __init__(self, spec, entries, slots, device):
+        self.spec, self.entries = spec, entries
+        self.data = torch.zeros((entries, slots) + tuple(spec.shape), dtype=getattr(torch, spec.dtype),
+                                device=device)
+
+
+class Cache:
+    """``kv_specs[i]`` / ``state_specs[i]`` describe cache entry i (None: the entry keeps none).
+
+    max_tokens  the most tokens live sequences hold together, each sequence rounded up to 64
+    max_sequence_length  the longest a single sequence may get (the position encoding's limit)
+    """
+
+    def __init__(self, kv_specs, state_specs, max_tokens, max_sequence_length, dtype, device,
+                 max_slots=None):
+        if max_tokens <= 0:
+            raise ValueError("max_tokens must be positive")
+        n_blocks = (max_tokens + BLOCK - 1) // BLOCK
+        self.dtype, self.device = dtype, device
+        self.max_tokens = n_blocks * BLOCK
+        self.max_sequence_length = min(max_sequence_length, self.max_tokens)
+        self.max_blocks = (self.max_sequence_length + BLOCK - 1) // BLOCK
+        self.max_slots = max_slots if max_slots is not None else min(n_blocks, 4096)
+        self.kv_groups, self.kv_entry = [], {}
+        by_spec = {}
+        for entry, spec in enumerate(kv_specs):
+            if spec is None:
+                continue
+            by_spec.setdefault(spec, []).append(entry)
+        for spec, entries in by_spec.items():
+            group = KVGroup(spec, len(entries), n_blocks, dtype, device)
+            for index, entry in enumerate(entries):
+                self.kv_entry[entry] = (len(self.kv_groups), index)
+            self.kv_groups.append(group)
+        self.state_groups, self.state_entry = [], {}
+        by_spec = {}
+        for entry, spec in enumerate(state_specs):
+            if spec is None:
+                continue
+            by_spec.setdefault(spec, []).append(entry)
+        for spec, entries in by_spec.items():
+            group = StateGroup(spec, len(entries), self.max_slots, device)
+            for index, entry in enumerate(entries):
+                self.state_entry[entry] = (len(self.state_groups), index)
+            self.state_groups.append(group)
+        # one block table serves every group: the ledger runs a single list of block numbers
+        self.ledger = CacheLedger(1 if self.kv_groups else 0, n_blocks, self.max_slots, self.max_blocks)
+
+    # --- slots -----------------------------------------------------------------------------
+    def acquire(self):
+        slot = self.ledger.acquire()
+        for group in self.state_groups:
+            group.data[:, slot].zero_()
+        return slot
+
+    def release(self, slot):
+        self.ledger.release(slot)
+
+    def length(self, slot):
+        return self.ledger.lengths[slot]
+
+    def blocks(self, slot):
+        return self.ledger.held_blocks[0][slot] if self.kv_groups else []
+
+    # --- views -----------------------------------------------------------------------------
+    def kv_view(self, entry, block_table):
+        group, index = self.kv_entry[entry]
+        return self.kv_groups[group].view(index, block_table, self.max_blocks)
+
+    def state(self, entry):
+        """[slots, *shape] state of a cache entry."""
+        group, index = self.state_entry[entry]
+        return self.state_groups[group].data[index]
+
+    def bytes(self):
+        total = sum(g.keys.numel() * g.keys.element_size() * 2 for g in self.kv_groups)
+        return total + sum(g.data.numel() * g.data.element_size() for g in self.state_groups)

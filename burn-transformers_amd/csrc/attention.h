@@ -1,0 +1,22 @@
+// Arguments of the attention kernels (plain and MFMA); mirrored by a ctypes.Structure.
+#pragma once
+
+#include "common.h"
+
+struct AttnArgs {
+  const void* q;        // [tokens][ldq]; head j at columns j * head_dim
+  int64_t ldq;
+  void* out;            // [tokens][ldo]
+  int64_t ldo;
+  const int* tok_seq;   // [tokens]
+  const int* tok_pos;   // [tokens]
+  const int* seq_off;   // [n_seqs + 1] first token of each sequence in the step
+  const int* seq_start; // [n_seqs] position of that first token
+  KvView kv;
+  int q_heads;
+  int n_tokens;
+  int n_seqs;
+  int max_count;        // most tokens any sequence brings in this step
+  int window;           // 0 = all earlier keys
+  float scale;
+};

@@ -1,0 +1,103 @@
+// Shared device helpers for the gfx950 kernels: element types, vector types,
+// the paged key/value addressing and wave/block reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define BT_EXPORT extern "C" __attribute__((visibility("default")))
+
+// Error codes returned by every entry point (0 = launched).
+#define BT_OK 0
+#define BT_REFUSED 1  // the sizes are outside what the kernel takes; see bt_last_error()
+#define BT_HIP_ERROR 2
+
+// Tokens per block of the paged key/value storage.  A key tile of 32 never straddles a block.
+#define BT_KV_BLOCK 64
+
+typedef __bf16 bf16_t;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+void bt_set_error(const char* fmt, ...);
+int bt_check_launch(const char* what);
+
+#define BT_REFUSE(...)            \
+  do {                            \
+    bt_set_error(__VA_ARGS__);    \
+    return BT_REFUSED;            \
+  } while (0)
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return (float)v; }
+
+template <typename T>
+__device__ __forceinline__ T from_float(float v);
+template <>
+__device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return (bf16_t)v; }  // round to nearest even
+
+// Geometry of one group of layers in the paged key/value storage.
+//   keys:   [layer][block][kv_head][BT_KV_BLOCK][head_dim]
+//   values: [layer][block][kv_head][BT_KV_BLOCK / 4][head_dim][4]   (four positions interleaved
+//           per channel, so that a lane reads four consecutive positions of one channel at once)
+// `blocks` is the table of the step's sequences: blocks[seq * max_blocks + position / BT_KV_BLOCK].
+struct KvView {
+  void* keys;            // base of the layer
+  void* values;          // base of the layer
+  const int* blocks;     // [n_seqs][max_blocks]
+  int max_blocks;
+  int kv_heads;
+  int head_dim;
+};
+
+__device__ __forceinline__ int64_t kv_block_base(const KvView& kv, int seq, int pos, int kv_head) {
+  int block = kv.blocks[(int64_t)seq * kv.max_blocks + pos / BT_KV_BLOCK];
+  return ((int64_t)block * kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * kv.head_dim);
+}
+// Element offset of key (pos, channel) inside its (block, head) plane.
+__device__ __forceinline__ int key_offset(int head_dim, int pos, int channel) {
+  return (pos % BT_KV_BLOCK) * head_dim + channel;
+}
+// Element offset of value (pos, channel) inside its (block, head) plane.
+__device__ __forceinline__ int value_offset(int head_dim, int pos, int channel) {
+  int p = pos % BT_KV_BLOCK;
+  return ((p >> 2) * head_dim + channel) * 4 + (p & 3);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Block-wide reductions for blocks of up to 1024 threads; `scratch` holds 32 floats of LDS.
+// Every thread gets the result.  Safe to call repeatedly with the same scratch.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < waves; ++w) total += scratch[w];
+  return total;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float top = scratch[0];
+  for (int w = 1; w < waves; ++w) top = fmaxf(top, scratch[w]);
+  return top;
+}

@@ -1,0 +1,430 @@
+// Core kernel module: the kernels every run needs, in plain form.
+//   * embedding gather (+ learned position table)
+//   * residual add + normalisation (32-bit statistics)
+//   * a plain tiled matrix product with true 32-bit multiply-accumulate
+//   * plain attention over the paged cache (one work-group per query row and head)
+//   * greedy and temperature sampling with log-probabilities
+// The 32-bit path of the model runs entirely on these; the bfloat16 path uses them for
+// everything that is not an MFMA kernel, and the tests use the matrix product and the
+// attention here as the slow twins of the MFMA kernels.
+
+#include "host.h"
+#include "epilogue.h"
+#include "attention.h"
+
+// ---------------------------------------------------------------------------------------------
+// Embedding: x[t] = table[ids[t]] (+ positions[pos[t]]), written as 32-bit residual stream.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,
+                             const T* __restrict__ table, const T* __restrict__ positions,
+                             float* __restrict__ out, int width) {
+  int t = blockIdx.x;
+  const T* row = table + (int64_t)ids[t] * width;
+  const T* prow = positions ? positions + (int64_t)pos[t] * width : nullptr;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float v = to_float(row[c]);
+    if (prow) v += to_float(prow[c]);
+    out[(int64_t)t * width + c] = v;
+  }
+}
+
+BT_EXPORT int bt_embed(void* stream, int dtype, const int* ids, const int* pos, const void* table,
+                       const void* positions, float* out, int tokens, int width) {
+  if (tokens <= 0) return BT_OK;
+  if (width <= 0) BT_REFUSE("embed: width %d must be positive", width);
+  dim3 grid(tokens), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, (hipStream_t)stream, ids, pos,
+                       (const float*)table, (const float*)positions, out, width);
+  else
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, ids, pos,
+                       (const bf16_t*)table, (const bf16_t*)positions, out, width);
+  return bt_check_launch("embed");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Residual add + normalisation.
+//   v = x[t] + sum_s delta[s][t] + bias          (t = rows ? rows[r] : r)
+//   x[t] = v                                     (if write_back)
+//   out[r] = norm(v) * gamma + beta              kind 0: (v - mean) / sqrt(var + eps)
+//                                                kind 1: v / sqrt(mean(v^2) + eps), no beta
+// Statistics in 32-bit with two passes over the row kept in LDS.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void add_norm_kernel(float* __restrict__ x, const float* __restrict__ delta, int n_delta,
+                                int64_t delta_stride, const float* __restrict__ bias,
+                                const float* __restrict__ gamma, const float* __restrict__ beta,
+                                float eps, int kind, T* __restrict__ out, const int* __restrict__ rows,
+                                int width, int write_back) {
+  extern __shared__ float row_buf[];
+  __shared__ float scratch[32];
+  int r = blockIdx.x;
+  int t = rows ? rows[r] : r;
+  float* xr = x + (int64_t)t * width;
+  float partial = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float v = xr[c];
+    for (int s = 0; s < n_delta; ++s) v += delta[s * delta_stride + (int64_t)t * width + c];
+    if (bias) v += bias[c];
+    row_buf[c] = v;
+    if (write_back) xr[c] = v;
+    partial += (kind == 0) ? v : v * v;
+  }
+  float total = block_sum(partial, scratch);
+  float mean = 0.f, rstd;
+  if (kind == 0) {
+    mean = total / (float)width;
+    float sq = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      float dlt = row_buf[c] - mean;
+      sq += dlt * dlt;
+    }
+    float var = block_sum(sq, scratch) / (float)width;
+    rstd = 1.0f / sqrtf(var + eps);
+  } else {
+    rstd = 1.0f / sqrtf(total / (float)width + eps);
+  }
+  if (out == nullptr) return;
+  T* orow = out + (int64_t)r * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float y = (row_buf[c] - mean) * rstd * gamma[c];
+    if (beta) y += beta[c];
+    orow[c] = from_float<T>(y);
+  }
+}
+
+BT_EXPORT int bt_add_norm(void* stream, int out_dtype, float* x, const float* delta, int n_delta,
+                          int64_t delta_stride, const float* bias, const float* gamma,
+                          const float* beta, float eps, int kind, void* out, const int* rows,
+                          int n_rows, int width, int write_back) {
+  if (n_rows <= 0) return BT_OK;
+  if (width <= 0 || width > 15360) BT_REFUSE("add_norm: width %d outside 1..15360 (the row is held in LDS)", width);
+  if (kind != 0 && kind != 1) BT_REFUSE("add_norm: unknown norm kind %d", kind);
+  dim3 grid(n_rows), block(256);
+  size_t lds = (size_t)width * sizeof(float);
+  if (out_dtype == 0)
+    hipLaunchKernelGGL(add_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, x, delta, n_delta,
+                       delta_stride, bias, gamma, beta, eps, kind, (float*)out, rows, width, write_back);
+  else
+    hipLaunchKernelGGL(add_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, x, delta, n_delta,
+                       delta_stride, bias, gamma, beta, eps, kind, (bf16_t*)out, rows, width, write_back);
+  return bt_check_launch("add_norm");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Plain matrix product C[M,N] = A[M,K] . W[N,K]^T with 32-bit FMA accumulation.
+// 64 x 64 tile, K in steps of 16, 256 threads with 4 x 4 outputs each.  Any M, N, K.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+gemm_plain_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W, int M, int N, int K,
+                  Epilogue epi) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Ws[16][64 + 4];
+  int tid = threadIdx.x;
+  int tx = tid & 15, ty = tid >> 4;
+  int m_base = blockIdx.y * 64, n_base = blockIdx.x * 64;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    // each thread loads 4 elements of A and of W: row = tid / 4 .. , column = (tid % 16)
+    for (int e = tid; e < 64 * 16; e += 256) {
+      int row = e >> 4, col = e & 15;
+      int k = k0 + col;
+      int m = m_base + row, n = n_base + row;
+      As[col][row] = (m < M && k < K) ? to_float(A[(int64_t)m * lda + k]) : 0.f;
+      Ws[col][row] = (n < N && k < K) ? to_float(W[(int64_t)n * K + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float a[4], w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int m = m_base + ty * 4 + i;
+    if (m < M) epilogue4<T>(epi, N, m, n_base + tx * 4, acc[i], 0);
+  }
+}
+
+int bt_check_epilogue(const Epilogue& e, int N, const char* who) {
+  if (e.mode < 0 || e.mode > 3) BT_REFUSE("%s: unknown epilogue mode %d", who, e.mode);
+  if (e.out == nullptr) BT_REFUSE("%s: epilogue has no output", who);
+  if (e.mode == EPI_QKV) {
+    if (e.kv.head_dim <= 0 || e.kv.head_dim % 16 != 0)
+      BT_REFUSE("%s: head size %d must be a multiple of 16", who, e.kv.head_dim);
+    if (e.n_q % 16 != 0 || e.n_kv != e.kv.kv_heads * e.kv.head_dim || e.n_q + 2 * e.n_kv != N)
+      BT_REFUSE("%s: fused projection of %d columns does not split into %d query and 2 x %d key/value columns",
+                who, N, e.n_q, e.n_kv);
+    if (!e.tok_seq || !e.tok_pos || !e.kv.blocks || !e.kv.keys || !e.kv.values)
+      BT_REFUSE("%s: the key/value scatter needs token and cache tables", who);
+  }
+  return BT_OK;
+}
+
+BT_EXPORT int bt_gemm_plain(void* stream, int dtype, const void* A, int64_t lda, const void* W, int M,
+                            int N, int K, const Epilogue* epi) {
+  if (M <= 0) return BT_OK;
+  if (N <= 0 || K <= 0) BT_REFUSE("gemm_plain: N %d and K %d must be positive", N, K);
+  int rc = bt_check_epilogue(*epi, N, "gemm_plain");
+  if (rc) return rc;
+  dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL(gemm_plain_kernel<float>, grid, block, 0, (hipStream_t)stream, (const float*)A, lda,
+                       (const float*)W, M, N, K, *epi);
+  else
+    hipLaunchKernelGGL(gemm_plain_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, (const bf16_t*)A,
+                       lda, (const bf16_t*)W, M, N, K, *epi);
+  return bt_check_launch("gemm_plain");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Plain attention over the paged cache.  One work-group per (token, query head).
+//   scores s_k = scale * (q . key_k) for keys lo <= k <= pos, lo = max(0, pos - window + 1)
+//   out = sum_k softmax(s)_k value_k, softmax in 32-bit with a running maximum over chunks.
+// Keys beyond the token's own position are never read.
+// ---------------------------------------------------------------------------------------------
+#define PLAIN_CHUNK 1024
+
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+attention_plain_kernel(AttnArgs a) {
+  __shared__ float qs[256];
+  __shared__ float ps[PLAIN_CHUNK];
+  __shared__ float scratch[32];
+  int t = blockIdx.x, head = blockIdx.y;
+  int hd = a.kv.head_dim;
+  int group = a.q_heads / a.kv.kv_heads;
+  int kv_head = head / group;
+  int seq = a.tok_seq[t], pos = a.tok_pos[t];
+  const T* q = static_cast<const T*>(a.q) + (int64_t)t * a.ldq + head * hd;
+  for (int c = threadIdx.x; c < hd; c += blockDim.x) qs[c] = to_float(q[c]);
+  __syncthreads();
+  int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  float run_max = -INFINITY, run_sum = 0.f, acc = 0.f;  // acc: channel threadIdx.x (< hd)
+  const T* keys = static_cast<const T*>(a.kv.keys);
+  const T* values = static_cast<const T*>(a.kv.values);
+  for (int c0 = lo; c0 <= pos; c0 += PLAIN_CHUNK) {
+    int n = pos + 1 - c0 < PLAIN_CHUNK ? pos + 1 - c0 : PLAIN_CHUNK;
+    float local_max = -INFINITY;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      int k = c0 + i;
+      const T* kr = keys + kv_block_base(a.kv, seq, k, kv_head) + key_offset(hd, k, 0);
+      float s = 0.f;
+      for (int c = 0; c < hd; ++c) s = fmaf(qs[c], to_float(kr[c]), s);
+      s *= a.scale;
+      ps[i] = s;
+      local_max = fmaxf(local_max, s);
+    }
+    float chunk_max = block_max(local_max, scratch);
+    float new_max = fmaxf(run_max, chunk_max);
+    float rescale = (run_max == -INFINITY) ? 0.f : expf(run_max - new_max);
+    float local_sum = 0.f;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      float p = expf(ps[i] - new_max);
+      ps[i] = p;
+      local_sum += p;
+    }
+    float chunk_sum = block_sum(local_sum, scratch);
+    run_sum = run_sum * rescale + chunk_sum;
+    run_max = new_max;
+    __syncthreads();
+    if ((int)threadIdx.x < hd) {
+      acc *= rescale;
+      for (int i = 0; i < n; ++i) {
+        int k = c0 + i;
+        const T* vr = values + kv_block_base(a.kv, seq, k, kv_head);
+        acc = fmaf(ps[i], to_float(vr[value_offset(hd, k, threadIdx.x)]), acc);
+      }
+    }
+    __syncthreads();
+  }
+  if ((int)threadIdx.x < hd) {
+    T* o = static_cast<T*>(a.out) + (int64_t)t * a.ldo + head * hd;
+    o[threadIdx.x] = from_float<T>(run_sum > 0.f ? acc / run_sum : 0.f);
+  }
+}
+
+int bt_check_attention(const AttnArgs& a, const char* who) {
+  int hd = a.kv.head_dim;
+  if (hd <= 0 || hd % 16 != 0 || hd > 256) BT_REFUSE("%s: head size %d must be a multiple of 16 up to 256", who, hd);
+  if (a.kv.kv_heads <= 0 || a.q_heads <= 0 || a.q_heads % a.kv.kv_heads != 0)
+    BT_REFUSE("%s: %d query heads cannot share %d key/value heads", who, a.q_heads, a.kv.kv_heads);
+  if (a.window < 0) BT_REFUSE("%s: window %d must not be negative", who, a.window);
+  if (!a.q || !a.out || !a.tok_seq || !a.tok_pos || !a.seq_off || !a.seq_start || !a.kv.blocks ||
+      !a.kv.keys || !a.kv.values)
+    BT_REFUSE("%s: missing operand", who);
+  return BT_OK;
+}
+
+BT_EXPORT int bt_attention_plain(void* stream, int dtype, const AttnArgs* args) {
+  if (args->n_tokens <= 0) return BT_OK;
+  int rc = bt_check_attention(*args, "attention_plain");
+  if (rc) return rc;
+  dim3 grid(args->n_tokens, args->q_heads), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL(attention_plain_kernel<float>, grid, block, 0, (hipStream_t)stream, *args);
+  else
+    hipLaunchKernelGGL(attention_plain_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *args);
+  return bt_check_launch("attention_plain");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Copies of keys and values between plain [tokens][kv_heads * head_dim] rows and the paged cache
+// (used by mixers that do not go through the fused projection, and by tests that read the cache).
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void kv_copy_kernel(T* __restrict__ k_rows, T* __restrict__ v_rows, int64_t ld,
+                               const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                               KvView kv, int to_cache) {
+  int t = blockIdx.x;
+  int seq = tok_seq[t], pos = tok_pos[t];
+  int hd = kv.head_dim;
+  T* keys = static_cast<T*>(kv.keys);
+  T* values = static_cast<T*>(kv.values);
+  for (int c = threadIdx.x; c < kv.kv_heads * hd; c += blockDim.x) {
+    int head = c / hd, channel = c % hd;
+    int64_t base = kv_block_base(kv, seq, pos, head);
+    int64_t ko = base + key_offset(hd, pos, channel), vo = base + value_offset(hd, pos, channel);
+    if (to_cache) {
+      keys[ko] = k_rows[(int64_t)t * ld + c];
+      values[vo] = v_rows[(int64_t)t * ld + c];
+    } else {
+      k_rows[(int64_t)t * ld + c] = keys[ko];
+      v_rows[(int64_t)t * ld + c] = values[vo];
+    }
+  }
+}
+
+BT_EXPORT int bt_kv_copy(void* stream, int dtype, void* k_rows, void* v_rows, int64_t ld,
+                         const int* tok_seq, const int* tok_pos, const KvView* kv, int tokens,
+                         int to_cache) {
+  if (tokens <= 0) return BT_OK;
+  if (kv->head_dim <= 0 || kv->head_dim % 4 != 0) BT_REFUSE("kv_copy: head size %d must be a multiple of 4", kv->head_dim);
+  dim3 grid(tokens), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL(kv_copy_kernel<float>, grid, block, 0, (hipStream_t)stream, (float*)k_rows,
+                       (float*)v_rows, ld, tok_seq, tok_pos, *kv, to_cache);
+  else
+    hipLaunchKernelGGL(kv_copy_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, (bf16_t*)k_rows,
+                       (bf16_t*)v_rows, ld, tok_seq, tok_pos, *kv, to_cache);
+  return bt_check_launch("kv_copy");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Sampling.  One work-group per row of 32-bit logits [rows][vocab].
+//   greedy: lowest index of the maximum; log-probability = log_softmax(z)[id]
+//   sample: p = softmax(z / T); id = #{k : c_k < u * c_last} with c the running sum of p in
+//           index order, u = ((mix(seed + gamma * (index + 1)) >> 41) + 0.5) / 2^23,
+//           index = first_draw + (draw_rows ? draw_rows[row] : row); log-probability of the
+//           tempered distribution.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t splitmix64(uint64_t seed, uint64_t index) {
+  uint64_t v = seed + 0x9E3779B97F4A7C15ull * (index + 1ull);
+  v = (v ^ (v >> 30)) * 0xBF58476D1CE4E5B9ull;
+  v = (v ^ (v >> 27)) * 0x94D049BB133111EBull;
+  return v ^ (v >> 31);
+}
+
+#define SAMPLE_THREADS 256
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int sample, float temperature,
+              uint64_t seed, uint64_t first_draw, const int* __restrict__ draw_rows,
+              int* __restrict__ ids, float* __restrict__ logp) {
+  __shared__ float scratch[32];
+  __shared__ float seg_sum[SAMPLE_THREADS];
+  __shared__ int best_index[SAMPLE_THREADS / 64];
+  __shared__ float best_value[SAMPLE_THREADS / 64];
+  __shared__ int chosen;
+  int row = blockIdx.x, tid = threadIdx.x;
+  const float* z = logits + (int64_t)row * ld;
+  // the logits are divided by the temperature only when sampling
+  float divisor = sample ? temperature : 1.0f;
+
+  // maximum and its lowest index
+  float top = -INFINITY;
+  int arg = 0x7fffffff;
+  for (int k = tid; k < vocab; k += SAMPLE_THREADS) {
+    float v = z[k] / divisor;
+    if (v > top) { top = v; arg = k; }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    float ov = __shfl_xor(top, o, 64);
+    int oa = __shfl_xor(arg, o, 64);
+    if (ov > top || (ov == top && oa < arg)) { top = ov; arg = oa; }
+  }
+  if ((tid & 63) == 0) { best_value[tid >> 6] = top; best_index[tid >> 6] = arg; }
+  __syncthreads();
+  top = best_value[0]; arg = best_index[0];
+  for (int w = 1; w < SAMPLE_THREADS / 64; ++w) {
+    if (best_value[w] > top || (best_value[w] == top && best_index[w] < arg)) { top = best_value[w]; arg = best_index[w]; }
+  }
+
+  // each thread owns one contiguous segment of the vocabulary, so that prefix sums run in index order
+  int seg = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  int lo = tid * seg, hi = lo + seg < vocab ? lo + seg : vocab;
+  float mine = 0.f;
+  for (int k = lo; k < hi; ++k) mine += expf(z[k] / divisor - top);
+  seg_sum[tid] = mine;
+  float total = block_sum(mine, scratch);  // also orders the seg_sum writes before the reads below
+
+  int pick = arg;
+  if (sample) {
+    if (tid == 0) {
+      float u = (float)(((double)(splitmix64(seed, first_draw + (uint64_t)(draw_rows ? draw_rows[row] : row)) >> 41) + 0.5) / 8388608.0);
+      float running = 0.f;
+      for (int t = 0; t < SAMPLE_THREADS; ++t) running += seg_sum[t];   // realised total in index order
+      float threshold = u * running;
+      float before = 0.f;
+      int owner = SAMPLE_THREADS - 1;
+      for (int t = 0; t < SAMPLE_THREADS; ++t) {
+        if (before + seg_sum[t] >= threshold) { owner = t; break; }
+        before += seg_sum[t];
+      }
+      int olo = owner * seg, ohi = olo + seg < vocab ? olo + seg : vocab;
+      int k = olo;
+      float c = before;
+      for (; k < ohi; ++k) {
+        c += expf(z[k] / divisor - top);
+        if (!(c < threshold)) break;
+      }
+      if (k >= vocab) k = vocab - 1;
+      chosen = k;
+    }
+    __syncthreads();
+    pick = chosen;
+  }
+  if (tid == 0) {
+    ids[row] = pick;
+    logp[row] = z[pick] / divisor - top - logf(total);
+  }
+}
+
+BT_EXPORT int bt_sample(void* stream, const float* logits, int64_t ld, int rows, int vocab, int sample,
+                        float temperature, uint64_t seed, uint64_t first_draw, const int* draw_rows,
+                        int* ids, float* logp) {
+  if (rows <= 0) return BT_OK;
+  if (vocab <= 0) BT_REFUSE("sample: vocabulary %d must be positive", vocab);
+  if (sample && !(temperature > 0.f)) BT_REFUSE("sample: temperature %g must be positive", (double)temperature);
+  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, logits, ld,
+                     vocab, sample, temperature, seed, first_draw, draw_rows, ids, logp);
+  return bt_check_launch("sample");
+}

@@ -1,0 +1,200 @@
+"""The engine: a model, its cache and the ONE step function that everything above it uses
+(generation, replay, benchmarks).
+
+    engine = Engine(model, max_tokens=4096)
+    slot = engine.open()                            # a sequence's handle
+    logits = engine.step([(slot, [5, 17, 3])], want=[[0, 2]])   # float32 [2, vocab]
+    logits = engine.step([(slot, [9])])             # one more token, logits of it
+    engine.close(slot)                              # gives the slot and its blocks back
+
+A step runs exactly the tokens it is given, as one packed batch without padding, against what
+earlier steps left in the cache, and returns the logits of the wanted places.  Sequences of a
+step may bring different numbers of tokens and stand at different lengths; whole prompts,
+chunks of prompts and single tokens all take this path (the reference's forward_cached does
+the same behind prefill and decode, src/models/llama/model/decode.rs:630-684).  Everything is
+validated before anything changes, lengths advance only after the forward pass was launched
+without error (decode.rs:38-41).
+
+Steps in which every sequence brings one token are replayed from a HIP graph per batch size:
+such a step is hundreds of short kernels, and launching them one by one costs more than
+running them.
+"""
+
+import numpy as np
+import torch
+
+from ..cache.storage import Cache
+from .step import BufferPool, Step, StepLayout, StepPlan
+
+_PINNED_RING = 4
+
+
+class StepError(ValueError):
+    """The step was refused; the cache is as it was."""
+
+
+class Engine:
+    def __init__(self, model, max_tokens, max_slots=None, graphs=True):
+        self.model = model
+        self.device, self.dtype = model.device, model.dtype
+        self.cache = Cache(model.kv_specs, model.state_specs, max_tokens, model.max_positions,
+                           model.dtype, model.device, max_slots)
+        self.pool = BufferPool(self.device)
+        self.use_graphs = graphs
+        self._meta = None                  # device int32 buffer of eager steps
+        self._pinned = []                  # ring of (pinned int32 tensor, event)
+        self._pinned_next = 0
+        self._graphs = {}                  # n_seqs -> dict(graph, meta, logits, generation)
+        self._seen_decode = set()
+        self.steps_run = 0
+        self.graph_replays = 0
+
+    # --- sequences -------------------------------------------------------------------------
+    def open(self):
+        """A slot for a new sequence."""
+        return self.cache.acquire()
+
+    def close(self, slot):
+        """Ends a sequence: its slot and its blocks can be used again."""
+        self.cache.release(slot)
+
+    def length(self, slot):
+        return self.cache.length(slot)
+
+    # --- the step function -----------------------------------------------------------------
+    def plan(self, entries, want=None):
+        """Validates a step and lays its tables out on the host.  Changes nothing."""
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        ledger = self.cache.ledger
+        slots, starts, counts, ids = [], [], [], []
+        for slot, tokens in entries:
+            if not ledger.live(slot):
+                raise StepError(f"slot {slot} is not open")
+            if slot in slots:
+                raise StepError(f"slot {slot} appears twice in one step")
+            tokens = np.asarray(tokens, dtype=np.int64).reshape(-1)
+            if tokens.size == 0:
+                raise StepError(f"slot {slot} brings no token; leave idle sequences out of the step")
+            if tokens.min() < 0 or tokens.max() >= self.model.vocab_size:
+                raise StepError(f"token ids of slot {slot} lie in {tokens.min()}..={tokens.max()}, "
+                                f"expected token values in 0..{self.model.vocab_size}")
+            start = ledger.lengths[slot]
+            limit = min(self.model.max_positions, self.cache.max_sequence_length)
+            if start + tokens.size > limit:
+                raise StepError(f"slot {slot} would reach {start + tokens.size} tokens, "
+                                f"the limit is {limit}")
+            slots.append(slot)
+            starts.append(start)
+            counts.append(int(tokens.size))
+            ids.append(tokens)
+        offsets = np.concatenate([[0], np.cumsum(counts)])
+        if want is None:
+            wanted = [int(offsets[i + 1] - 1) for i in range(len(entries))]
+        else:
+            if len(want) != len(entries):
+                raise StepError("`want` needs one list of places per sequence")
+            wanted = []
+            for i, places in enumerate(want):
+                for place in places:
+                    if not (0 <= place < counts[i]):
+                        raise StepError(f"wanted place {place} of slot {slots[i]} is outside its "
+                                        f"{counts[i]} tokens")
+                    wanted.append(int(offsets[i] + place))
+        new_lengths = {s: st + c for s, st, c in zip(slots, starts, counts)}
+        try:
+            ledger.check_growth(new_lengths)
+        except RuntimeError as error:
+            raise StepError(str(error)) from error
+        # block rows are read after the reservation, in `step`
+        return dict(slots=slots, starts=starts, counts=counts, ids=np.concatenate(ids), wanted=wanted,
+                    new_lengths=new_lengths)
+
+    def step(self, entries, want=None):
+        """Runs one step; returns float32 logits [wanted places, vocab] on the GPU, valid until the
+        next step.  ``entries``: [(slot, token ids)], ``want``: per entry the places among its
+        tokens whose logits are wanted (default: each entry's last token)."""
+        checked = self.plan(entries, want)
+        ledger = self.cache.ledger
+        for slot, length in checked["new_lengths"].items():
+            ledger.reserve(slot, length)
+        plan = StepPlan(checked["slots"], checked["starts"], checked["counts"], checked["ids"],
+                        checked["wanted"], [self.cache.blocks(s) for s in checked["slots"]],
+                        self.cache.max_blocks)
+        if not checked["wanted"]:
+            logits = self._run_eager(plan, want_logits=False)
+        elif plan.decode and self.use_graphs and plan.layout.rows == plan.n_seqs and \
+                checked["wanted"] == list(range(plan.n_seqs)):
+            logits = self._run_decode_graph(plan)
+        else:
+            logits = self._run_eager(plan)
+        for slot, length in checked["new_lengths"].items():
+            ledger.commit(slot, length)
+        self.steps_run += 1
+        return logits
+
+    # --- running ---------------------------------------------------------------------------
+    def _upload(self, host, device_meta):
+        """One copy of the step's tables to the GPU through a pinned staging buffer."""
+        if len(self._pinned) < _PINNED_RING:
+            self._pinned.append([torch.empty(max(host.size, 4096), dtype=torch.int32, pin_memory=True),
+                                 torch.cuda.Event()])
+        entry = self._pinned[self._pinned_next % len(self._pinned)]
+        self._pinned_next += 1
+        entry[1].synchronize()                       # the copy that last used this buffer is done
+        if entry[0].numel() < host.size:
+            entry[0] = torch.empty(host.size * 2, dtype=torch.int32, pin_memory=True)
+        entry[0][:host.size].numpy()[:] = host
+        device_meta[:host.size].copy_(entry[0][:host.size], non_blocking=True)
+        entry[1].record()
+
+    def _run_eager(self, plan, want_logits=True):
+        if self._meta is None or self._meta.numel() < plan.layout.total:
+            self._meta = torch.empty(max(plan.layout.total * 2, 4096), dtype=torch.int32, device=self.device)
+        self._upload(plan.host, self._meta)
+        step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
+        if not want_logits:
+            self._forward_without_readout(step)
+            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        return self.model.forward(step, self.cache)
+
+    def _forward_without_readout(self, step):
+        """A step whose logits nobody wants still has to fill the cache."""
+        model = self.model
+        from ..parts import Memory
+        stream = model.embedding.embed(step)
+        for entry in model.schedule:
+            memory = Memory(self.cache, entry.cache, entry.writes, step) if entry.cache is not None else None
+            model.blocks[entry.layer].forward(stream, step, memory)
+
+    def _run_decode_graph(self, plan):
+        key = plan.n_seqs
+        held = self._graphs.get(key)
+        if held is not None and held["generation"] != self.pool.generation:
+            held = None                                   # a workspace moved: the graph is stale
+            del self._graphs[key]
+        if held is None:
+            if key not in self._seen_decode:              # first time: run eagerly, which also sizes the workspaces
+                self._seen_decode.add(key)
+                return self._run_eager(plan)
+            held = self._capture(plan)
+        self._upload(plan.host, held["meta"])
+        held["graph"].replay()
+        self.graph_replays += 1
+        return held["logits"]
+
+    def _capture(self, plan):
+        meta = torch.empty(plan.layout.total, dtype=torch.int32, device=self.device)
+        self._upload(plan.host, meta)
+        step = Step(plan.layout, meta, self.pool, self.dtype, plan)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        self.pool.frozen = True
+        try:
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(step, self.cache)
+        finally:
+            self.pool.frozen = False
+        held = dict(graph=graph, meta=meta, logits=logits, generation=self.pool.generation)
+        self._graphs[plan.n_seqs] = held
+        return held

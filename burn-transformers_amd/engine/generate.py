@@ -1,0 +1,123 @@
+"""The generation loop above the step function.
+
+Requests (prompts of unequal length) are taken in order and packed into batches that fit the
+cache; each batch is prefilled in one step (or in chunks), then decoded one token per step.
+A sequence that ends leaves the batch at once and gives its slot back; the next batch uses
+the slots again.  One readback per step brings the chosen ids and their log-probabilities to
+the host (src/generation/causal.rs:118-211 is the reference's loop; its rows stay in the
+batch with a mask, here they leave it).
+"""
+
+import math
+
+import torch
+
+from ..cache.ledger import BLOCK
+from ..sampling.config import GenerationConfig, GenerationError
+from ..sampling.sampler import Sampler
+from ..sampling.tracker import GenerationTracker, required_capacity
+
+
+def _rounded(tokens):
+    return (tokens + BLOCK - 1) // BLOCK * BLOCK
+
+
+def plan_batches(prompt_lengths, max_new_tokens, max_tokens, max_slots, sequence_limit, batch_size=None):
+    """Splits requests, in order, into batches whose sequences fit the cache together.
+    Pure bookkeeping; raises if a single request cannot fit."""
+    batches, current, used = [], [], 0
+    for index, length in enumerate(prompt_lengths):
+        if length <= 0:
+            raise GenerationError(f"prompt {index} is empty")
+        need = required_capacity(length, max_new_tokens)
+        if need > sequence_limit:
+            raise GenerationError(
+                f"prompt {index}: {length} prompt tokens + {max_new_tokens} new tokens need {need} positions, "
+                f"the limit is {sequence_limit}")
+        if _rounded(need) > max_tokens:
+            raise GenerationError(f"prompt {index} needs {_rounded(need)} cache tokens, the cache holds {max_tokens}")
+        full = (batch_size is not None and len(current) >= batch_size) or len(current) >= max_slots
+        if current and (full or used + _rounded(need) > max_tokens):
+            batches.append(current)
+            current, used = [], 0
+        current.append(index)
+        used += _rounded(need)
+    if current:
+        batches.append(current)
+    return batches
+
+
+def prefill_chunks(prompt_lengths, chunk):
+    """For chunked prefill: a list of steps, each a list of (row, begin, end) token ranges.  Rows
+    that have run out of prompt are simply absent from later chunks."""
+    if chunk is None:
+        return [[(row, 0, n) for row, n in enumerate(prompt_lengths)]]
+    if chunk <= 0:
+        raise GenerationError("prefill_chunk_size must be greater than zero")
+    steps = []
+    for begin in range(0, max(prompt_lengths), chunk):
+        steps.append([(row, begin, min(begin + chunk, n)) for row, n in enumerate(prompt_lengths) if n > begin])
+    return steps
+
+
+def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None):
+    """Runs one batch that starts together to completion; returns its GeneratedSequences."""
+    tracker = GenerationTracker(config, [len(p) for p in prompts])
+    sampler = Sampler(config, len(prompts), engine.device)
+    slots = [engine.open() for _ in prompts]
+    open_rows = set(range(len(prompts)))
+    try:
+        logits = torch.empty((len(prompts), engine.model.vocab_size), dtype=torch.float32, device=engine.device)
+        for chunk in prefill_chunks([len(p) for p in prompts], prefill_chunk):
+            entries = [(slots[row], prompts[row][begin:end]) for row, begin, end in chunk]
+            # each row's logits are wanted from the chunk in which its prompt ends
+            final = [row for row, _, end in chunk if end == len(prompts[row])]
+            want = [[end - begin - 1] if end == len(prompts[row]) else [] for row, begin, end in chunk]
+            chunk_logits = engine.step(entries, want)
+            if final:
+                logits.index_copy_(0, torch.tensor(final, device=engine.device), chunk_logits)
+        live = list(range(len(prompts)))
+        while True:
+            ids, logps = sampler.select(logits, live)
+            next_live, next_entries = [], []
+            for row, token, logp in zip(live, ids, logps):
+                if not math.isfinite(logp):
+                    raise GenerationError(f"row {row}: the selected token has a non-finite log-probability")
+                reason = tracker.push(row, token, logp)
+                if on_token is not None:
+                    on_token(row, token, logp, reason)
+                if reason is None:
+                    next_live.append(row)
+                    next_entries.append((slots[row], [token]))
+                else:                                   # the sequence leaves the batch; its slot is free again
+                    engine.close(slots[row])
+                    open_rows.discard(row)
+            if not next_live:
+                break
+            live = next_live
+            logits = engine.step(next_entries)
+    finally:
+        for row in open_rows:
+            engine.close(slots[row])
+    return tracker.sequences
+
+
+def generate(engine, prompts, config=None, prefill_chunk=None, batch_size=None, on_token=None):
+    """Generates for every prompt (lists of token ids); returns GeneratedSequences in order."""
+    config = config or GenerationConfig()
+    config.validate(engine.model.vocab_size)
+    prompts = [list(p) for p in prompts]
+    if not prompts:
+        raise GenerationError("no prompts")
+    limit = min(engine.model.max_positions, engine.cache.max_sequence_length)
+    batches = plan_batches([len(p) for p in prompts], config.max_new_tokens, engine.cache.max_tokens,
+                           engine.cache.max_slots, limit, batch_size)
+    results = [None] * len(prompts)
+    for batch in batches:
+        callback = None
+        if on_token is not None:
+            callback = lambda row, token, logp, reason, batch=batch: on_token(batch[row], token, logp, reason)
+        for index, sequence in zip(batch, generate_batch(engine, [prompts[i] for i in batch], config,
+                                                         prefill_chunk, callback)):
+            results[index] = sequence
+    return results

@@ -1,0 +1,101 @@
+"""Builds a model from a plan and a weight store, and runs its forward pass for one step.
+
+The model is what the registry hands out for an architecture name: embedding, the layers made
+of registered parts, the schedule in which they run, the final norm and the readout.  It holds
+no sizes of its own; everything comes from the plan (and so from config.json).
+"""
+
+from ..config.base import read_config_json
+from ..config.registry import resolve_family
+from ..kernels import library as K
+from ..parts import Memory, lookup
+from ..weights.loader import compute_dtype, load_checkpoint, store_from_tensors
+
+
+def build_part(role, spec, store):
+    missing = [name for name in spec.tensors.values() if name not in store]
+    if missing:
+        raise KeyError(f"{role} {spec.kind!r} asks for tensors the weight store does not hold: {missing}")
+    return lookup(role, spec.kind)(spec.params, {r: store[name] for r, name in spec.tensors.items()})
+
+
+class CausalLM:
+    def __init__(self, plan, store, config=None, family=None):
+        self.plan, self.store, self.config, self.family = plan, store, config, family
+        self.dtype, self.device = store.dtype, store.device
+        self.width, self.vocab_size, self.max_positions = plan.width, plan.vocab_size, plan.max_positions
+        self.embedding = build_part("embedding", plan.embedding, store)
+        self.blocks = []
+        for layer in plan.layers:
+            block_class = lookup("block", layer.block)
+            unknown = set(layer.parts) - set(block_class.ROLES)
+            absent = set(block_class.ROLES) - set(layer.parts)
+            if unknown or absent:
+                raise ValueError(f"block {layer.block!r} takes parts {sorted(block_class.ROLES)}, "
+                                 f"the plan gives {sorted(layer.parts)}")
+            self.blocks.append(block_class({name: build_part(block_class.ROLES[name], spec, store)
+                                            for name, spec in layer.parts.items()}))
+        self.final_norm = build_part("norm", plan.final_norm, store)
+        self.readout = build_part("readout", plan.readout, store)
+        self.schedule = list(plan.schedule)
+        self._check_schedule()
+        head_dims = sorted({d for block in self.blocks for d in block.parts["mixer"].head_dims()})
+        K.prepare(self.dtype, head_dims)
+
+    def _check_schedule(self):
+        """Every cache entry has exactly one writer, which runs before any reader, and readers keep
+        what the writer keeps."""
+        writers = {}
+        for position, entry in enumerate(self.schedule):
+            if not (0 <= entry.layer < len(self.blocks)):
+                raise ValueError(f"schedule entry {position} names layer {entry.layer}, "
+                                 f"the model has {len(self.blocks)}")
+            if entry.cache is None:
+                continue
+            mixer = self.blocks[entry.layer].parts["mixer"]
+            specs = (mixer.kv_spec(), mixer.state_spec())
+            if entry.writes:
+                if entry.cache in writers:
+                    raise ValueError(f"cache entry {entry.cache} has two writers in the schedule")
+                writers[entry.cache] = specs
+            elif entry.cache not in writers:
+                raise ValueError(f"schedule entry {position} reads cache entry {entry.cache} before it is written")
+            elif writers[entry.cache] != specs:
+                raise ValueError(f"schedule entry {position} reads cache entry {entry.cache}, "
+                                 f"whose keys and values have another shape")
+        self.cache_entries = max(writers) + 1 if writers else 0
+        self.kv_specs = [writers.get(i, (None, None))[0] for i in range(self.cache_entries)]
+        self.state_specs = [writers.get(i, (None, None))[1] for i in range(self.cache_entries)]
+
+    def forward(self, step, cache):
+        """Logits (float32 [len(step.sel_rows), vocab]) of the step's wanted rows."""
+        stream = self.embedding.embed(step)
+        for entry in self.schedule:
+            memory = Memory(cache, entry.cache, entry.writes, step) if entry.cache is not None else None
+            self.blocks[entry.layer].forward(stream, step, memory)
+        hidden = self.final_norm.apply(stream, step, rows=step.sel_rows)
+        return self.readout.logits(hidden, step)
+
+
+def _device(device):
+    import torch
+    K.require_gpu()
+    return torch.device(device if device is not None else "cuda:0")
+
+
+def load_model(model_dir, dtype="bfloat16", device=None):
+    """The model of a folder with config.json and safetensors weights; the class of model is the
+    one config.json names."""
+    config_json = read_config_json(model_dir)
+    family = resolve_family(config_json)
+    config = family.config_class.from_dict(config_json)
+    store = load_checkpoint(model_dir, family.contract(config), compute_dtype(dtype), _device(device))
+    return CausalLM(family.plan(config), store, config, family)
+
+
+def model_from_tensors(config_json, tensors, dtype="bfloat16", device=None):
+    """The same model from in-memory tensors under checkpoint names (random weights, tests)."""
+    family = resolve_family(config_json)
+    config = family.config_class.from_dict(config_json)
+    store = store_from_tensors(tensors, family.contract(config), compute_dtype(dtype), _device(device))
+    return CausalLM(family.plan(config), store, config, family)

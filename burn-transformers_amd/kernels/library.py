@@ -1,0 +1,225 @@
+"""ctypes bindings of the HIP kernel modules.
+
+Every function here launches kernels on torch's current HIP stream and takes torch tensors
+on the GPU.  There is no fallback: a module that cannot be built or loaded raises, and a size
+that a kernel does not take raises :class:`KernelError` with the kernel's own message.
+"""
+
+import ctypes
+import threading
+
+import torch  # imported first: the kernel libraries bind to the HIP runtime torch has loaded
+
+from . import build
+
+FLOAT32, BFLOAT16 = 0, 1
+DTYPE_CODES = {torch.float32: FLOAT32, torch.bfloat16: BFLOAT16}
+
+EPI_STORE, EPI_ACT, EPI_F32, EPI_QKV = 0, 1, 2, 3
+ACTIVATIONS = {"gelu_tanh": 0, "gelu_erf": 1}
+NORM_KINDS = {"layer_norm": 0, "rms_norm": 1}
+KV_BLOCK = 64
+
+_c_int, _c_i64, _c_ptr, _c_float, _c_u64 = (ctypes.c_int, ctypes.c_int64, ctypes.c_void_p,
+                                           ctypes.c_float, ctypes.c_uint64)
+
+
+class KernelError(RuntimeError):
+    """A kernel refused its operands or a launch failed."""
+
+
+class KvView(ctypes.Structure):
+    """One layer of one group of the paged key/value storage, as the kernels see it."""
+    _fields_ = [("keys", _c_ptr), ("values", _c_ptr), ("blocks", _c_ptr),
+                ("max_blocks", _c_int), ("kv_heads", _c_int), ("head_dim", _c_int)]
+
+
+class Epilogue(ctypes.Structure):
+    _fields_ = [("mode", _c_int), ("act", _c_int), ("bias", _c_ptr), ("out", _c_ptr),
+                ("ldo", _c_i64), ("split_stride", _c_i64), ("n_q", _c_int), ("n_kv", _c_int),
+                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView)]
+
+
+class AttnArgs(ctypes.Structure):
+    _fields_ = [("q", _c_ptr), ("ldq", _c_i64), ("out", _c_ptr), ("ldo", _c_i64),
+                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("seq_off", _c_ptr), ("seq_start", _c_ptr),
+                ("kv", KvView), ("q_heads", _c_int), ("n_tokens", _c_int), ("n_seqs", _c_int),
+                ("max_count", _c_int), ("window", _c_int), ("scale", _c_float)]
+
+
+_modules = {}
+_lock = threading.Lock()
+
+
+def _module(name):
+    with _lock:
+        lib = _modules.get(name)
+        if lib is None:
+            path = build.ensure(name)
+            try:
+                lib = ctypes.CDLL(path)
+            except OSError as error:
+                raise RuntimeError(f"cannot load the kernel library {path}: {error}") from error
+            lib.bt_last_error.restype = ctypes.c_char_p
+            _modules[name] = lib
+        return lib
+
+
+def _check(lib, code):
+    if code != 0:
+        raise KernelError(lib.bt_last_error().decode())
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(tensor):
+    return None if tensor is None else tensor.data_ptr()
+
+
+def loaded_modules():
+    return sorted(_modules)
+
+
+def require_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("burn_transformers_amd runs on an AMD GPU only (no HIP device is visible); "
+                           "there is no CPU path")
+
+
+def prepare(dtype, head_dims=()):
+    """Builds and loads what a model of this dtype and these head sizes needs."""
+    _module("core")
+    if dtype == torch.bfloat16:
+        _module("gemm_bf16")
+        for size in head_dims:
+            _module(f"attention_bf16_hd{size}")
+
+
+# --- epilogues -------------------------------------------------------------------------------
+
+def epilogue_store(out, bias=None):
+    return Epilogue(mode=EPI_STORE, bias=_ptr(bias), out=out.data_ptr(), ldo=out.stride(0))
+
+
+def epilogue_act(out, activation, bias=None):
+    return Epilogue(mode=EPI_ACT, act=ACTIVATIONS[activation], bias=_ptr(bias), out=out.data_ptr(),
+                    ldo=out.stride(0))
+
+
+def epilogue_f32(out, bias=None):
+    """``out`` is float32 [splits, M, N] (or [M, N] for one split)."""
+    split_stride = out.stride(0) if out.dim() == 3 else 0
+    return Epilogue(mode=EPI_F32, bias=_ptr(bias), out=out.data_ptr(), ldo=out.stride(-2),
+                    split_stride=split_stride)
+
+
+def epilogue_qkv(q_out, n_q, n_kv, kv_view, tok_seq, tok_pos, bias=None):
+    return Epilogue(mode=EPI_QKV, bias=_ptr(bias), out=q_out.data_ptr(), ldo=q_out.stride(0), n_q=n_q,
+                    n_kv=n_kv, tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), kv=kv_view)
+
+
+# --- kernels ---------------------------------------------------------------------------------
+
+def embed(ids, positions, table, position_table, out):
+    """out[t] = table[ids[t]] (+ position_table[positions[t]]); out is the float32 stream."""
+    lib = _module("core")
+    _check(lib, lib.bt_embed(_c_ptr(_stream()), DTYPE_CODES[table.dtype], _c_ptr(ids.data_ptr()),
+                             _c_ptr(_ptr(positions)), _c_ptr(table.data_ptr()), _c_ptr(_ptr(position_table)),
+                             _c_ptr(out.data_ptr()), _c_int(ids.numel()), _c_int(table.shape[1])))
+
+
+def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None, rows=None,
+             write_back=True):
+    """x[t] += sum(delta[:, t]) + bias (kept when ``write_back``); out[r] = norm(x[t]) * gamma + beta
+    with t = rows[r] if rows is given else r.  ``out`` may be None (only the add)."""
+    lib = _module("core")
+    width = x.shape[1]
+    if delta is None:
+        n_delta, stride = 0, 0
+    elif delta.dim() == 3:
+        n_delta, stride = delta.shape[0], delta.stride(0)
+    else:
+        n_delta, stride = 1, 0
+    n_rows = rows.numel() if rows is not None else x.shape[0]
+    out_dtype = DTYPE_CODES[out.dtype] if out is not None else FLOAT32
+    _check(lib, lib.bt_add_norm(
+        _c_ptr(_stream()), _c_int(out_dtype), _c_ptr(x.data_ptr()), _c_ptr(_ptr(delta)), _c_int(n_delta),
+        _c_i64(stride), _c_ptr(_ptr(bias)), _c_ptr(_ptr(gamma)), _c_ptr(_ptr(beta)), _c_float(eps),
+        _c_int(NORM_KINDS[kind]), _c_ptr(_ptr(out)), _c_ptr(_ptr(rows)), _c_int(n_rows), _c_int(width),
+        _c_int(1 if write_back else 0)))
+
+
+def gemm(a, w, epilogue, splits=1, impl="auto"):
+    """C = a . w^T handed to ``epilogue``.  a: [M, K] (rows may be strided), w: [N, K] contiguous.
+
+    impl: "auto" (float32 -> plain; bfloat16 -> skinny up to 64 rows, else tile), or one of
+    "plain", "tile", "skinny" to force a kernel.
+    """
+    m, k = a.shape
+    n = w.shape[0]
+    if w.shape[1] != k or a.stride(1) != 1 or not w.is_contiguous() or a.dtype != w.dtype:
+        raise KernelError(f"gemm: operands [{m},{k}] {a.dtype} and [{n},{w.shape[1]}] {w.dtype} do not fit")
+    dtype = DTYPE_CODES[a.dtype]
+    if impl == "auto":
+        impl = "plain" if dtype == FLOAT32 else ("skinny" if m <= 64 else "tile")
+    args = (_c_ptr(a.data_ptr()), _c_i64(a.stride(0)), _c_ptr(w.data_ptr()), _c_int(m), _c_int(n), _c_int(k),
+            ctypes.byref(epilogue))
+    if impl == "plain":
+        if splits != 1:
+            raise KernelError("gemm: the plain kernel does not split K")
+        lib = _module("core")
+        _check(lib, lib.bt_gemm_plain(_c_ptr(_stream()), _c_int(dtype), *args))
+        return
+    if dtype != BFLOAT16:
+        raise KernelError(f"gemm: the {impl} kernel takes bfloat16 only")
+    lib = _module("gemm_bf16")
+    fn = lib.bt_gemm_tile_bf16 if impl == "tile" else lib.bt_gemm_skinny_bf16
+    _check(lib, fn(_c_ptr(_stream()), *args, _c_int(splits)))
+
+
+def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
+                   scale, window=0):
+    return AttnArgs(q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0),
+                    tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), seq_off=seq_off.data_ptr(),
+                    seq_start=seq_start.data_ptr(), kv=kv_view, q_heads=q_heads, n_tokens=q.shape[0],
+                    n_seqs=n_seqs, max_count=max_count, window=window or 0, scale=scale)
+
+
+def attention(args, dtype, decode, impl="auto"):
+    """Attention of the step's tokens over the cache.  impl: "auto", "plain" or "mfma"."""
+    code = DTYPE_CODES[dtype]
+    if impl == "auto":
+        impl = "plain" if code == FLOAT32 else "mfma"
+    if impl == "plain":
+        lib = _module("core")
+        _check(lib, lib.bt_attention_plain(_c_ptr(_stream()), _c_int(code), ctypes.byref(args)))
+        return
+    if code != BFLOAT16:
+        raise KernelError("attention: the MFMA kernels take bfloat16 only")
+    lib = _module(f"attention_bf16_hd{args.kv.head_dim}")
+    fn = lib.bt_attention_decode_bf16 if decode else lib.bt_attention_prefill_bf16
+    _check(lib, fn(_c_ptr(_stream()), ctypes.byref(args)))
+
+
+def kv_copy(k_rows, v_rows, tok_seq, tok_pos, kv_view, to_cache):
+    """Copies [tokens, kv_heads * head_dim] rows into the paged cache, or back out of it."""
+    lib = _module("core")
+    _check(lib, lib.bt_kv_copy(_c_ptr(_stream()), _c_int(DTYPE_CODES[k_rows.dtype]), _c_ptr(k_rows.data_ptr()),
+                               _c_ptr(v_rows.data_ptr()), _c_i64(k_rows.stride(0)), _c_ptr(tok_seq.data_ptr()),
+                               _c_ptr(tok_pos.data_ptr()), ctypes.byref(kv_view), _c_int(k_rows.shape[0]),
+                               _c_int(1 if to_cache else 0)))
+
+
+def sample(logits, ids, logp, temperature=None, seed=0, first_draw=0, draw_rows=None):
+    """Greedy (temperature None) or temperature sampling of each row of float32 logits.  Row r uses
+    draw number first_draw + (draw_rows[r] if draw_rows is given else r) of the seed's stream."""
+    lib = _module("core")
+    rows, vocab = logits.shape
+    sampling = temperature is not None
+    _check(lib, lib.bt_sample(_c_ptr(_stream()), _c_ptr(logits.data_ptr()), _c_i64(logits.stride(0)),
+                              _c_int(rows), _c_int(vocab), _c_int(1 if sampling else 0),
+                              _c_float(temperature if sampling else 1.0), _c_u64(seed & (2 ** 64 - 1)),
+                              _c_u64(first_draw & (2 ** 64 - 1)), _c_ptr(_ptr(draw_rows)), _c_ptr(ids.data_ptr()),
+                              _c_ptr(logp.data_ptr())))

@@ -1,0 +1,70 @@
+"""Causal self-attention with grouped heads over the paged cache.
+
+Parameters (all from the plan): width, heads, kv_heads, head_dim, scale (multiplies q.k),
+window (0 = every earlier key), causal.  Tensors: a fused projection ``qkv_weight`` held
+[heads*head_dim + 2*kv_heads*head_dim, width] with its bias, and ``out_weight`` [width,
+heads*head_dim] with its bias.
+
+One step: the fused projection's epilogue writes the queries to a buffer and scatters the new
+keys and values straight into the cache at each token's position; the attention kernel then
+reads the cache (prefill: tiled, online softmax; decode: one query per head, keys split over
+the waves); the output projection leaves 32-bit partial sums for the next norm to add.
+Formulas: src/attention.rs:481-513 (projections), src/attention/dispatch.rs:314-328, 365-367,
+390-406 (scaled scores, exclusion by -inf, 32-bit softmax), src/attention.rs:882-897 (merge and
+output projection).
+"""
+
+from ..cache.storage import KVSpec
+from ..kernels import library as K
+from .base import Delta, Mixer, split_count
+from .registry import register
+
+
+@register("mixer", "attention")
+class CausalSelfAttention(Mixer):
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        p = params
+        self.width, self.heads, self.kv_heads = p["width"], p["heads"], p["kv_heads"]
+        self.head_dim, self.scale, self.window = p["head_dim"], float(p["scale"]), int(p.get("window") or 0)
+        if not p.get("causal", True):
+            raise ValueError("attention: only causal attention runs from a cache")
+        if self.head_dim % 16 != 0:
+            raise ValueError(f"attention: head size {self.head_dim} must be a multiple of 16")
+        if self.heads % self.kv_heads != 0:
+            raise ValueError(f"attention: {self.heads} query heads cannot share {self.kv_heads} key/value heads")
+        self.n_q, self.n_kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
+        self.qkv_weight, self.qkv_bias = tensors["qkv_weight"], tensors.get("qkv_bias")
+        self.out_weight, self.out_bias = tensors["out_weight"], tensors.get("out_bias")
+        if tuple(self.qkv_weight.shape) != (self.n_q + 2 * self.n_kv, self.width):
+            raise ValueError(f"attention: fused projection is {tuple(self.qkv_weight.shape)}, "
+                             f"expected {(self.n_q + 2 * self.n_kv, self.width)}")
+        if tuple(self.out_weight.shape) != (self.width, self.n_q):
+            raise ValueError(f"attention: output projection is {tuple(self.out_weight.shape)}, "
+                             f"expected {(self.width, self.n_q)}")
+
+    def kv_spec(self):
+        return KVSpec(self.kv_heads, self.head_dim, self.window)
+
+    def head_dims(self):
+        return (self.head_dim,)
+
+    def forward(self, h, step, memory):
+        tokens = h.shape[0]
+        kv = memory.kv()
+        q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
+        if memory.writes:
+            K.gemm(h, self.qkv_weight,
+                   K.epilogue_qkv(q, self.n_q, self.n_kv, kv, step.tok_seq, step.tok_pos, self.qkv_bias))
+        else:   # the keys and values of another layer are read; only the queries are projected
+            bias = self.qkv_bias[:self.n_q] if self.qkv_bias is not None else None
+            K.gemm(h, self.qkv_weight[:self.n_q], K.epilogue_store(q, bias))
+        mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
+        args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
+                                self.heads, step.n_seqs, step.max_count, self.scale, self.window)
+        K.attention(args, step.dtype, step.decode)
+        splits = split_count(tokens, self.width, self.n_q) if step.dtype_is_bf16 else 1
+        partials = step.buffer("attention.delta", splits * tokens, self.width, "float32").view(
+            splits, tokens, self.width)
+        K.gemm(mixed, self.out_weight, K.epilogue_f32(partials), splits=splits)
+        return Delta(partials, self.out_bias)

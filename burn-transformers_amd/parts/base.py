@@ -1,0 +1,125 @@
+"""The interfaces the parts of a layer meet, and the residual stream they work on.
+
+  Norm         apply(stream, step, rows=None) -> normalised activations [tokens, width]
+  Mixer        forward(h, step, memory) -> Delta         (attention here; anything that mixes tokens)
+               kv_spec() / state_spec() say what it keeps in the cache, per token / per sequence
+  FeedForward  forward(h, step) -> Delta
+  Embedding    embed(step) -> ResidualStream             (token table and position encoding)
+  Readout      logits(h, step) -> float32 [rows, vocab]
+  Block        forward(stream, step, memory)             (the arrangement of the parts above)
+
+No part knows which model it is in: it gets its sizes and constants as parameters and its
+tensors by role from the weight store.
+
+The residual stream is kept in float32 in both precisions, and a part's contribution is not
+added at once: it is left as a :class:`Delta` (32-bit partial sums of a matrix product, plus a
+bias) that the next norm adds while it reads the stream anyway.  That saves one pass over the
+stream per part and lets a matrix product split its K range without a reduction pass.
+"""
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from ..kernels import library as K
+
+
+@dataclass
+class Delta:
+    """A contribution to the residual stream that has not been added yet:
+    sum(partials, dim 0) + bias.  partials: float32 [splits, tokens, width]."""
+    partials: torch.Tensor
+    bias: Optional[torch.Tensor] = None
+
+
+class ResidualStream:
+    def __init__(self, x):
+        self.x = x              # float32 [tokens, width]
+        self.pending = None     # Delta or None
+
+    def add(self, delta):
+        if self.pending is not None:
+            self.flush()
+        self.pending = delta
+
+    def flush(self):
+        """Adds what is pending without normalising anything."""
+        if self.pending is not None:
+            K.add_norm(self.x, None, None, None, 0.0, delta=self.pending.partials, bias=self.pending.bias)
+            self.pending = None
+
+
+class Memory:
+    """What a mixer gets of the cache for one run of its layer."""
+
+    def __init__(self, cache, entry, writes, step):
+        self.cache, self.entry, self.writes, self.step = cache, entry, writes, step
+
+    def kv(self):
+        """Kernel view of this entry's keys and values with the step's block table."""
+        return self.cache.kv_view(self.entry, self.step.block_table)
+
+    def state(self):
+        """[slots, *shape] per-sequence state of this entry; rows ``step.slots`` are the step's."""
+        return self.cache.state(self.entry)
+
+
+class Part:
+    def __init__(self, params, tensors):
+        self.params, self.tensors = params, tensors
+
+
+class Norm(Part):
+    def apply(self, stream, step, rows=None):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def kv_spec(self):
+        return None
+
+    def state_spec(self):
+        return None
+
+    def head_dims(self):
+        """Head sizes for which attention kernels must be built."""
+        return ()
+
+    def forward(self, h, step, memory):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h, step):
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def embed(self, step):
+        raise NotImplementedError
+
+
+class Readout(Part):
+    def logits(self, h, step):
+        raise NotImplementedError
+
+
+class Block:
+    def __init__(self, parts):
+        self.parts = parts
+
+    def forward(self, stream, step, memory):
+        raise NotImplementedError
+
+
+def split_count(rows, columns, k):
+    """How many ways a residual-writing product splits its K range in decode: few output columns
+    give too few work-groups to pull a weight matrix through HBM at full rate."""
+    if rows > 64:
+        return 1
+    tiles = (columns + 15) // 16
+    splits = 1
+    while tiles * splits < 512 and splits < 8 and k // (splits * 2) >= 256:
+        splits *= 2
+    return splits

@@ -1,0 +1,44 @@
+"""Normalisations over the channel axis, with 32-bit statistics in both precisions.
+
+layer_norm: y = (x - mean) / sqrt(var + eps) * weight + bias, var the population variance
+            (src/models/gpt2/model.rs:8, 143-148).
+rms_norm:   y = x / sqrt(mean(x^2) + eps) * weight   (src/normalization.rs:158-171).
+
+``apply`` first adds what is pending on the residual stream, in the same pass.
+"""
+
+from ..kernels import library as K
+from .base import Norm
+from .registry import register
+
+
+class _KernelNorm(Norm):
+    KIND = None
+
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        self.width, self.eps = params["width"], float(params["eps"])
+        self.weight, self.bias = tensors["weight"], tensors.get("bias")
+        if tuple(self.weight.shape) != (self.width,):
+            raise ValueError(f"{self.KIND}: scale is {tuple(self.weight.shape)}, expected {(self.width,)}")
+
+    def apply(self, stream, step, rows=None):
+        count = rows.numel() if rows is not None else stream.x.shape[0]
+        out = step.buffer("norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)
+        pending = stream.pending
+        K.add_norm(stream.x, out, self.weight, self.bias, self.eps, self.KIND,
+                   delta=pending.partials if pending else None, bias=pending.bias if pending else None,
+                   rows=rows, write_back=rows is None)
+        if rows is None:
+            stream.pending = None
+        return out
+
+
+@register("norm", "layer_norm")
+class LayerNorm(_KernelNorm):
+    KIND = "layer_norm"
+
+
+@register("norm", "rms_norm")
+class RMSNorm(_KernelNorm):
+    KIND = "rms_norm"

@@ -1,0 +1,22 @@
+"""Readout: logits = h . table^T in float32, no bias; the table is [vocab, width] and may be
+the token table itself (src/models/gpt2/model.rs:500-513, src/operations.rs:675-728)."""
+
+from ..kernels import library as K
+from .base import Readout
+from .registry import register
+
+
+@register("readout", "linear_readout")
+class LinearReadout(Readout):
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        self.width, self.vocab_size = params["width"], params["vocab_size"]
+        self.weight = tensors["weight"]
+        if tuple(self.weight.shape) != (self.vocab_size, self.width):
+            raise ValueError(f"readout: table is {tuple(self.weight.shape)}, expected "
+                             f"{(self.vocab_size, self.width)}")
+
+    def logits(self, h, step):
+        out = step.buffer("readout.logits", h.shape[0], self.vocab_size, "float32")
+        K.gemm(h, self.weight, K.epilogue_f32(out))
+        return out

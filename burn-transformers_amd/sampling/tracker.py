@@ -1,0 +1,85 @@
+"""Per-sequence bookkeeping of a generation: emitted tokens, log-probabilities and why a
+sequence ended.  Pure Python; the generation loop asks it after every token.
+
+Rules (src/generation.rs:1277-1422, src/generation/bookkeeping.rs:177-296):
+  * an end-of-sequence token is emitted, then the sequence ends (EndOfSequence);
+  * otherwise the longest stop sequence that is a suffix of the emitted tokens ends it
+    (StopSequence; ties go to the first configured); the matched tokens stay emitted;
+  * otherwise reaching max_new_tokens ends it (Length);
+  * before min_new_tokens neither end-of-sequence nor stop sequences are looked at.
+"""
+
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+
+@dataclass
+class FinishReason:
+    kind: str                          # "eos", "stop" or "length"
+    token_id: Optional[int] = None     # eos
+    index: Optional[int] = None        # stop: which configured sequence
+    length: Optional[int] = None       # stop: its length
+
+    def __str__(self):
+        if self.kind == "eos":
+            return f"EndOfSequence(token_id={self.token_id})"
+        if self.kind == "stop":
+            return f"StopSequence(index={self.index}, length={self.length})"
+        return "Length"
+
+
+@dataclass
+class GeneratedSequence:
+    prompt_length: int
+    token_ids: List[int] = field(default_factory=list)
+    log_probabilities: List[float] = field(default_factory=list)
+    finish_reason: Optional[FinishReason] = None
+
+
+def stop_decision(config, emitted):
+    """Why a sequence whose emitted tokens are ``emitted`` ends now, or None."""
+    count = len(emitted)
+    if count >= config.min_new_tokens:
+        if emitted and emitted[-1] in config.eos_token_ids:
+            return FinishReason("eos", token_id=emitted[-1])
+        best = None
+        for index, sequence in enumerate(config.stop_sequences):
+            n = len(sequence)
+            if n <= count and emitted[count - n:] == list(sequence) and (best is None or n > best[1]):
+                best = (index, n)
+        if best is not None:
+            return FinishReason("stop", index=best[0], length=best[1])
+    if count >= config.max_new_tokens:
+        return FinishReason("length")
+    return None
+
+
+class GenerationTracker:
+    def __init__(self, config, prompt_lengths):
+        self.config = config
+        self.sequences = [GeneratedSequence(n) for n in prompt_lengths]
+
+    def push(self, row, token, log_probability):
+        """Records a token of a live row; returns its finish reason if it ends now."""
+        sequence = self.sequences[row]
+        if sequence.finish_reason is not None:
+            raise RuntimeError(f"row {row} has already finished")
+        sequence.token_ids.append(int(token))
+        sequence.log_probabilities.append(float(log_probability))
+        sequence.finish_reason = stop_decision(self.config, sequence.token_ids)
+        return sequence.finish_reason
+
+    def finished(self, row):
+        return self.sequences[row].finish_reason is not None
+
+    def live_rows(self):
+        return [i for i, s in enumerate(self.sequences) if s.finish_reason is None]
+
+    def all_finished(self):
+        return all(s.finish_reason is not None for s in self.sequences)
+
+
+def required_capacity(prompt_length, max_new_tokens):
+    """Positions a sequence occupies: the last generated token is returned but never fed back
+    (src/generation/bookkeeping.rs:736-747)."""
+    return prompt_length + max_new_tokens - 1

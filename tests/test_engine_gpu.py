@@ -1,0 +1,260 @@
+"""The engine against the plain implementation: every way of cutting and batching the same
+requests gives the same logits, in float32 and in bfloat16."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import burn_transformers_amd as bt  # noqa: E402
+import plain_gpt2 as plain  # noqa: E402
+from model_helpers import CONFIGS, model_folder, plain_logits, prompts_for, tolerance  # noqa: E402
+
+DTYPES = ["float32", "bfloat16"]
+_models = {}
+
+
+def engine_for(name, dtype, max_tokens=2048, gain=1.0, **kw):
+    key = (name, dtype, gain)
+    if key not in _models:
+        folder, _, _ = model_folder(name, gain)
+        _models[key] = bt.load_model(folder, dtype=dtype, device="cuda:0")
+    return bt.Engine(_models[key], max_tokens=max_tokens, **kw)
+
+
+def check(got, want, dtype, what):
+    got = got.detach().cpu().double()
+    err = float((got - want).abs().max())
+    assert torch.isfinite(got).all(), what
+    assert err <= tolerance(dtype, want), f"{what}: max abs error {err} > {tolerance(dtype, want)}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,lengths", [("A", [5, 11, 17, 100]), ("B", [1, 23, 64, 65, 150])])
+def test_each_request_alone_and_whole(name, dtype, lengths):
+    engine = engine_for(name, dtype)
+    for ids in prompts_for(name, lengths):
+        slot = engine.open()
+        logits = engine.step([(slot, ids)], want=[list(range(len(ids)))])
+        check(logits, plain_logits(name, ids), dtype, f"{name} whole {len(ids)}")
+        engine.close(slot)
+    engine.cache.ledger.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,length", [("A", 100), ("B", 150), ("B", 33)])
+def test_last_32_tokens_one_by_one(name, dtype, length):
+    engine = engine_for(name, dtype)
+    ids = prompts_for(name, [length], seed=3)[0]
+    want = plain_logits(name, ids)
+    slot = engine.open()
+    head = length - 32
+    rows = []
+    if head > 0:
+        rows.append(engine.step([(slot, ids[:head])], want=[list(range(head))]).clone())
+    for t in range(max(head, 0), length):
+        rows.append(engine.step([(slot, [ids[t]])]).clone())
+    check(torch.cat(rows), want, dtype, f"{name} decode tail of {length}")
+    assert engine.graph_replays > 0
+    engine.close(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_of_a_sequence(name, dtype):
+    """Token by token from the very first token."""
+    engine = engine_for(name, dtype)
+    ids = prompts_for(name, [20], seed=4)[0]
+    slot = engine.open()
+    rows = [engine.step([(slot, [t])]).clone() for t in ids]
+    check(torch.cat(rows), plain_logits(name, ids), dtype, f"{name} from the first token")
+    engine.close(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,chunk,lengths", [("A", 7, [1, 23, 40]), ("B", 64, [150, 70, 3]), ("B", 5, [9])])
+def test_chunked_prompts(name, dtype, chunk, lengths):
+    engine = engine_for(name, dtype)
+    prompts = prompts_for(name, lengths, seed=5)
+    slots = [engine.open() for _ in prompts]
+    got = [[] for _ in prompts]
+    for begin in range(0, max(lengths), chunk):
+        rows = [i for i, p in enumerate(prompts) if len(p) > begin]
+        entries = [(slots[i], prompts[i][begin:begin + chunk]) for i in rows]
+        want = [list(range(len(e[1]))) for e in entries]
+        logits = engine.step(entries, want).clone()
+        at = 0
+        for i, e in zip(rows, entries):
+            got[i].append(logits[at:at + len(e[1])])
+            at += len(e[1])
+    for i, p in enumerate(prompts):
+        check(torch.cat(got[i]), plain_logits(name, p), dtype, f"{name} chunks of {chunk}, prompt {i}")
+    for s in slots:
+        engine.close(s)
+    engine.cache.ledger.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_unequal_batches_one_after_another(name, dtype):
+    """Batches of unequal prompts, decoded with teacher forcing; shorter requests end earlier and
+    their slots are used again by the next batch, whose results must not see the old occupants."""
+    limit = CONFIGS[name][0]["n_positions"]
+    engine = engine_for(name, dtype, max_tokens=64 * 8)
+    batches = [[5, 70, 17], [64, 3, 90, 1], [33, 33], [100, 2, 65]]
+    seen_slots = []
+    for b, lengths in enumerate(batches):
+        totals = [min(n + 9 + 5 * i, limit) for i, n in enumerate(lengths)]
+        requests = prompts_for(name, totals, seed=10 + b)
+        slots = [engine.open() for _ in requests]
+        seen_slots.append(list(slots))
+        got = [[] for _ in requests]
+        logits = engine.step([(s, r[:n]) for s, r, n in zip(slots, requests, lengths)],
+                             want=[list(range(n)) for n in lengths]).clone()
+        at = 0
+        for i, n in enumerate(lengths):
+            got[i].append(logits[at:at + n])
+            at += n
+        live = list(range(len(requests)))
+        position = list(lengths)
+        while live:
+            entries = [(slots[i], [requests[i][position[i]]]) for i in live]
+            logits = engine.step(entries).clone()
+            for row, i in enumerate(live):
+                got[i].append(logits[row:row + 1])
+                position[i] += 1
+            for i in [i for i in live if position[i] >= totals[i]]:
+                engine.close(slots[i])            # ends earlier than the others
+                live.remove(i)
+        for i, r in enumerate(requests):
+            check(torch.cat(got[i]), plain_logits(name, r), dtype, f"{name} batch {b} request {i}")
+        engine.cache.ledger.check()
+    assert set(seen_slots[0]) & set(seen_slots[1]), "slots were not used again"
+    assert engine.cache.ledger.slots.available() == engine.cache.max_slots
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_reused_blocks_do_not_leak(dtype):
+    """A slot's blocks are poisoned with NaN after it is closed; the next occupant must not care."""
+    engine = engine_for("A", dtype, max_tokens=256)
+    first = prompts_for("A", [120], seed=20)[0]
+    slot = engine.open()
+    engine.step([(slot, first)])
+    engine.close(slot)
+    for group in engine.cache.kv_groups:
+        group.keys.fill_(float("nan"))
+        group.values.fill_(float("nan"))
+    ids = prompts_for("A", [50], seed=21)[0]
+    slot = engine.open()
+    rows = [engine.step([(slot, ids[:30])], want=[list(range(30))]).clone()]
+    rows += [engine.step([(slot, [t])]).clone() for t in ids[30:]]
+    check(torch.cat(rows), plain_logits("A", ids), dtype, "poisoned cache")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(dtype):
+    """Decoding far past several block edges, against whole-sequence logits."""
+    engine = engine_for("B", dtype)
+    ids = prompts_for("B", [192], seed=30)[0]
+    want = plain_logits("B", ids)
+    slot = engine.open()
+    rows = [engine.step([(slot, ids[:2])], want=[[0, 1]]).clone()]
+    rows += [engine.step([(slot, [t])]).clone() for t in ids[2:]]
+    check(torch.cat(rows), want, dtype, "long decode")
+
+
+def test_graph_and_eager_decoding_agree_bitwise():
+    ids = prompts_for("A", [40], seed=31)[0]
+    outs = []
+    for graphs in (True, False):
+        engine = engine_for("A", "bfloat16", graphs=graphs)
+        slot = engine.open()
+        rows = [engine.step([(slot, ids[:8])]).clone()]
+        rows += [engine.step([(slot, [t])]).clone() for t in ids[8:]]
+        outs.append(torch.cat(rows))
+        assert (engine.graph_replays > 0) == graphs
+    assert torch.equal(outs[0], outs[1])
+
+
+def test_refused_steps_change_nothing():
+    engine = engine_for("A", "float32", max_tokens=128)
+    slot = engine.open()
+    engine.step([(slot, [1, 2, 3])])
+    before = (engine.length(slot), list(engine.cache.blocks(slot)))
+    from burn_transformers_amd.engine.engine import StepError
+    with pytest.raises(StepError, match="token values in 0..1000"):
+        engine.step([(slot, [5, 1000])])
+    with pytest.raises(StepError, match="outside its"):
+        engine.step([(slot, [5])], want=[[1]])
+    with pytest.raises(StepError, match="limit"):
+        engine.step([(slot, [1] * 126)])
+    with pytest.raises(StepError, match="twice"):
+        engine.step([(slot, [1]), (slot, [2])])
+    other = engine.open()
+    with pytest.raises(StepError, match="blocks"):
+        engine.step([(other, [1] * 100)])          # 2 blocks needed, 1 free
+    assert (engine.length(slot), list(engine.cache.blocks(slot))) == before
+    assert engine.length(other) == 0 and not engine.cache.blocks(other)
+    engine.cache.ledger.check()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(name):
+    gain = 6.0
+    folder, config, weights = model_folder(name, gain)
+    prompts = prompts_for(name, [5, 11, 17], seed=40)
+    want = [plain.greedy(p, weights, config, 8) for p in prompts]
+    engine = engine_for(name, "float32", gain=gain)
+    got = bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=8))
+    assert [s.token_ids for s in got] == want
+    for sequence, prompt in zip(got, prompts):
+        assert sequence.prompt_length == len(prompt) and str(sequence.finish_reason) == "Length"
+        full = prompt + sequence.token_ids
+        ref = torch.log_softmax(plain.forward(full, weights, config), -1)
+        for i, (token, logp) in enumerate(zip(sequence.token_ids, sequence.log_probabilities)):
+            assert abs(logp - float(ref[len(prompt) - 1 + i, token])) < 1e-4
+    chunked = bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=8), prefill_chunk=7)
+    assert [s.token_ids for s in chunked] == want
+    # bfloat16 follows the same path; its tokens may leave the reference where logits nearly tie
+    engine16 = engine_for(name, "bfloat16", gain=gain)
+    got16 = bt.generate(engine16, prompts, bt.GenerationConfig(max_new_tokens=8))
+    same = sum(a == b for s, w in zip(got16, want) for a, b in zip(s.token_ids, w))
+    assert same >= 16
+    engine.cache.ledger.check()
+
+
+def test_sampling_end_of_sequence_and_batches():
+    folder, config, weights = model_folder("B", 6.0)
+    engine = engine_for("B", "float32", gain=6.0, max_tokens=64 * 3)
+    prompts = prompts_for("B", [1, 23, 9, 30, 2], seed=41)
+    cfg = bt.GenerationConfig(max_new_tokens=12, strategy="sample", temperature=0.8, seed=7)
+    first = bt.generate(engine, prompts, cfg, prefill_chunk=7, batch_size=2)
+    again = bt.generate(engine, prompts, cfg, batch_size=2)
+    assert [s.token_ids for s in first] == [s.token_ids for s in again]
+    other = bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=12, strategy="sample",
+                                                             temperature=0.8, seed=8), batch_size=2)
+    assert [s.token_ids for s in first] != [s.token_ids for s in other]
+    # every sampled token is the inverse-CDF choice of the plain implementation for its draw
+    for batch_start in (0, 2, 4):
+        rows = list(range(batch_start, min(batch_start + 2, len(prompts))))
+        for b, index in enumerate(rows):
+            full = prompts[index] + first[index].token_ids
+            logits = plain.forward(full, weights, config)
+            for s, token in enumerate(first[index].token_ids):
+                u = plain.interior_unit(plain.splitmix64(7, s * len(rows) + b))
+                z = logits[len(prompts[index]) - 1 + s]
+                p = torch.cumsum(torch.softmax(z / 0.8, -1), -1)
+                lo = float(p[token - 1]) if token else 0.0
+                assert lo - 1e-4 <= u <= float(p[token]) + 1e-4
+    # an end-of-sequence token ends its row, the others go on
+    greedy = bt.generate(engine, prompts[:3], bt.GenerationConfig(max_new_tokens=10))
+    eos = greedy[1].token_ids[3]
+    stopped = bt.generate(engine, prompts[:3], bt.GenerationConfig(max_new_tokens=10, eos_token_ids=[eos]))
+    cut = greedy[1].token_ids.index(eos) + 1
+    assert stopped[1].token_ids == greedy[1].token_ids[:cut]
+    assert str(stopped[1].finish_reason) == f"EndOfSequence(token_id={eos})"
+    for i in (0, 2):
+        if eos not in greedy[i].token_ids:
+            assert stopped[i].token_ids == greedy[i].token_ids
+    engine.cache.ledger.check()
+    assert engine.cache.ledger.slots.available() == engine.cache.max_slots

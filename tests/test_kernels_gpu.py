@@ -1,0 +1,266 @@
+"""Each kernel alone against a plain float64 reference, at sizes other than the engine's."""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from burn_transformers_amd.kernels import library as K  # noqa: E402
+from kernel_helpers import PagedCase, gelu_erf, gelu_tanh  # noqa: E402
+
+DEV = "cuda:0"
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rel_err(got, want):
+    got, want = got.detach().cpu().to(torch.float64), want.detach().cpu().to(torch.float64)
+    return float((got - want).abs().max() / (want.abs().max() + 1e-30))
+
+
+def operands(m, n, k, dtype, seed=0, lda=None):
+    gen = torch.Generator().manual_seed(seed)
+    lda = lda or k
+    a_full = (torch.randn(m, lda, generator=gen)).to(dtype).to(DEV)
+    a = a_full[:, :k]
+    w = (torch.randn(n, k, generator=gen) / math.sqrt(k)).to(dtype).to(DEV)
+    bias = torch.randn(n, generator=gen).to(DEV)
+    want = a.cpu().double() @ w.cpu().double().t()
+    return a, w, bias, want
+
+
+GEMM_CASES = [("plain", "float32", 1, 50, 24), ("plain", "float32", 70, 131, 40), ("plain", "bfloat16", 33, 67, 72),
+              ("tile", "bfloat16", 128, 128, 64), ("tile", "bfloat16", 200, 300, 136),
+              ("tile", "bfloat16", 300, 517, 1600), ("tile", "bfloat16", 65, 50257 // 16, 96),
+              ("skinny", "bfloat16", 1, 100, 136), ("skinny", "bfloat16", 7, 48, 1600),
+              ("skinny", "bfloat16", 16, 333, 72), ("skinny", "bfloat16", 17, 64, 320),
+              ("skinny", "bfloat16", 33, 1000, 64), ("skinny", "bfloat16", 64, 517, 6400)]
+
+
+@pytest.mark.parametrize("impl,dtype,m,n,k", GEMM_CASES)
+def test_gemm_epilogues(impl, dtype, m, n, k):
+    dt = DTYPES[dtype]
+    tol = 2e-6 if dtype == "float32" else 6e-3
+    a, w, bias, want = operands(m, n, k, dt, seed=m + n + k, lda=k + 8)
+    out = torch.full((m, n), float("nan"), dtype=dt, device=DEV)
+    K.gemm(a, w, K.epilogue_store(out, bias), impl=impl)
+    assert rel_err(out, want + bias.cpu().double()) < tol
+    for name, fn in (("gelu_tanh", gelu_tanh), ("gelu_erf", gelu_erf)):
+        out = torch.full((m, n), float("nan"), dtype=dt, device=DEV)
+        K.gemm(a, w, K.epilogue_act(out, name, bias), impl=impl)
+        assert rel_err(out, fn(want + bias.cpu().double())) < tol
+    out32 = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    K.gemm(a, w, K.epilogue_f32(out32), impl=impl)
+    assert rel_err(out32, want) < (2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k))
+
+
+@pytest.mark.parametrize("impl,m,n,k,splits", [("skinny", 5, 96, 1600, 4), ("skinny", 64, 50, 6400, 8),
+                                               ("skinny", 20, 1600, 320, 2), ("tile", 150, 200, 1600, 3)])
+def test_gemm_split_k_partials(impl, m, n, k, splits):
+    a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=splits)
+    parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl=impl)
+    assert rel_err(parts.sum(0), want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
+
+
+def test_gemm_refuses_what_it_cannot_take():
+    a, w, bias, _ = operands(4, 32, 20, torch.bfloat16)
+    out = torch.empty(4, 32, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(K.KernelError, match="multiples of 8"):
+        K.gemm(a, w, K.epilogue_store(out), impl="skinny")
+    a, w, bias, _ = operands(80, 32, 64, torch.bfloat16)
+    out = torch.empty(80, 32, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(K.KernelError, match="at most 64"):
+        K.gemm(a, w, K.epilogue_store(out), impl="skinny")
+    with pytest.raises(K.KernelError, match="partial sums"):
+        K.gemm(a, w, K.epilogue_store(out), impl="tile", splits=2)
+
+
+@pytest.mark.parametrize("impl,dtype,counts", [("plain", "float32", [3, 1, 70]), ("plain", "bfloat16", [5, 2]),
+                                               ("tile", "bfloat16", [100, 1, 37]), ("skinny", "bfloat16", [1, 1, 1]),
+                                               ("skinny", "bfloat16", [9, 30])])
+def test_fused_projection_scatters_into_the_cache(impl, dtype, counts):
+    dt = DTYPES[dtype]
+    q_heads, kv_heads, hd, width = 4, 2, 32, 72
+    totals = [c + 61 + 7 * i for i, c in enumerate(counts)]
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=1)
+    n_q, n_kv = q_heads * hd, kv_heads * hd
+    a, w, bias, want = operands(case.n_tokens, n_q + 2 * n_kv, width, dt, seed=9)
+    want = want + bias.cpu().double()
+    q = torch.full((case.n_tokens, n_q), float("nan"), dtype=dt, device=DEV)
+    before_k, before_v = case.read_back()
+    K.gemm(a, w, K.epilogue_qkv(q, n_q, n_kv, case.view(), case.tok_seq, case.tok_pos, bias), impl=impl)
+    after_k, after_v = case.read_back()
+    tol = 2e-6 if dtype == "float32" else 6e-3
+    assert rel_err(q, want[:, :n_q]) < tol
+    row, base = 0, 0
+    for total, count in zip(totals, counts):
+        new = slice(base + total - count, base + total)
+        old = slice(base, base + total - count)
+        assert rel_err(after_k[new], want[row:row + count, n_q:n_q + n_kv]) < tol
+        assert rel_err(after_v[new], want[row:row + count, n_q + n_kv:]) < tol
+        assert torch.equal(after_k[old], before_k[old]) and torch.equal(after_v[old], before_v[old])
+        row, base = row + count, base + total
+
+
+ATTN_CASES = [
+    # q_heads, kv_heads, head_dim, totals, counts, window
+    (2, 2, 16, [5, 11, 17], [5, 11, 17], 0),          # whole prompts
+    (3, 1, 48, [70, 130], [1, 1], 0),                 # decode, grouped heads, two blocks
+    (4, 2, 32, [200, 64, 65], [40, 64, 1], 0),        # chunks on non-empty caches, block edges
+    (2, 2, 64, [300, 129], [300, 2], 50),             # window
+    (5, 5, 80, [33], [33], 0),
+    (2, 1, 128, [260, 31], [1, 1], 100),              # decode with a window
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("q_heads,kv_heads,hd,totals,counts,window", ATTN_CASES)
+def test_attention_plain(dtype, q_heads, kv_heads, hd, totals, counts, window):
+    dt = DTYPES[dtype]
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=2, poison=True)
+    gen = torch.Generator().manual_seed(5)
+    q = torch.randn(case.n_tokens, q_heads * hd, generator=gen).to(dt).to(DEV)
+    out = torch.full((case.n_tokens, q_heads * hd), float("nan"), dtype=dt, device=DEV)
+    scale = 0.37 / math.sqrt(hd)
+    args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                            q_heads, len(totals), max(counts), scale, window)
+    K.attention(args, dt, decode=max(counts) == 1, impl="plain")
+    want = case.reference(q, q_heads, scale, window)
+    assert rel_err(out, want) < (3e-6 if dtype == "float32" else 8e-3)
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,hd,totals,counts,window", ATTN_CASES)
+def test_attention_mfma(q_heads, kv_heads, hd, totals, counts, window):
+    dt = torch.bfloat16
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=3, poison=True)
+    gen = torch.Generator().manual_seed(6)
+    q = torch.randn(case.n_tokens, q_heads * hd, generator=gen).to(dt).to(DEV)
+    scale = 0.37 / math.sqrt(hd)
+    want = case.reference(q, q_heads, scale, window)
+    kinds = [False] + ([True] if max(counts) == 1 else [])
+    for decode in kinds:
+        out = torch.full((case.n_tokens, q_heads * hd), float("nan"), dtype=dt, device=DEV)
+        args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                                q_heads, len(totals), max(counts), scale, window)
+        K.attention(args, dt, decode=decode, impl="mfma")
+        assert rel_err(out, want) < 1.2e-2, f"decode kernel={decode}"
+
+
+def test_attention_finds_one_far_key_among_hundreds():
+    """One key far back is made to dominate; an off-by-one in block or tile addressing loses it."""
+    dt = torch.bfloat16
+    hd, total = 64, 700
+    for target in (0, 63, 64, 333, 698):
+        case = PagedCase([total], [1], 1, hd, dt, DEV, seed=target)
+        q = torch.zeros(1, hd)
+        q[0, 3] = 8.0
+        case.k_rows[0][:] *= 0.05
+        case.k_rows[0][target, 3] = 8.0
+        seq = torch.zeros(total, dtype=torch.int32, device=DEV)
+        pos = torch.arange(total, dtype=torch.int32, device=DEV)
+        K.kv_copy(case.k_rows[0].to(DEV), case.v_rows[0].to(DEV), seq, pos, case.view(), True)
+        q = q.to(dt).to(DEV)
+        want = case.reference(q, 1, 1.0)
+        assert (want[0] - case.v_rows[0][target].double()).abs().max() < 1e-3
+        for impl, decode in (("plain", True), ("mfma", True), ("mfma", False)):
+            out = torch.empty(1, hd, dtype=dt, device=DEV)
+            args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                                    1, 1, 1, 1.0, 0)
+            K.attention(args, dt, decode=decode, impl=impl)
+            assert rel_err(out, want) < 1e-2, (target, impl, decode)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width,rows", [(64, 3), (96, 17), (1600, 5), (50, 2)])
+def test_add_norm(dtype, width, rows):
+    dt = DTYPES[dtype]
+    gen = torch.Generator().manual_seed(width)
+    x = (torch.randn(rows, width, generator=gen) * 2 + 0.5).to(DEV)
+    delta = torch.randn(3, rows, width, generator=gen).to(DEV)
+    bias = torch.randn(width, generator=gen).to(DEV)
+    gamma = (1 + 0.1 * torch.randn(width, generator=gen)).to(DEV)
+    beta = torch.randn(width, generator=gen).to(DEV)
+    total = x.double() + delta.double().sum(0) + bias.double()
+    want = torch.nn.functional.layer_norm(total, (width,), gamma.double(), beta.double(), 1e-3)
+    tol = 3e-6 if dtype == "float32" else 5e-3
+    xs = x.clone()
+    out = torch.empty(rows, width, dtype=dt, device=DEV)
+    K.add_norm(xs, out, gamma, beta, 1e-3, "layer_norm", delta=delta, bias=bias)
+    assert rel_err(out, want) < tol
+    assert rel_err(xs, total) < 1e-6
+    # selected rows: nothing is written back
+    pick = torch.tensor([rows - 1, 0], dtype=torch.int32, device=DEV)
+    xs = x.clone()
+    out = torch.empty(2, width, dtype=dt, device=DEV)
+    K.add_norm(xs, out, gamma, beta, 1e-3, "layer_norm", delta=delta, bias=bias, rows=pick, write_back=False)
+    assert rel_err(out, want[[rows - 1, 0]]) < tol
+    assert torch.equal(xs, x)
+    # root-mean-square norm, no shift
+    xs = x.clone()
+    out = torch.empty(rows, width, dtype=dt, device=DEV)
+    K.add_norm(xs, out, gamma, None, 1e-3, "rms_norm")
+    want = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-3) * gamma.double()
+    assert rel_err(out, want) < tol
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(dtype):
+    dt = DTYPES[dtype]
+    gen = torch.Generator().manual_seed(0)
+    table = torch.randn(37, 50, generator=gen).to(dt).to(DEV)
+    positions = torch.randn(20, 50, generator=gen).to(dt).to(DEV)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([19, 0, 3, 4, 7], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 50, dtype=torch.float32, device=DEV)
+    K.embed(ids, pos, table, positions, out)
+    assert torch.equal(out, table[ids.long()].float() + positions[pos.long()].float())
+    K.embed(ids, None, table, None, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+def test_greedy_takes_the_lowest_index_of_the_maximum():
+    gen = torch.Generator().manual_seed(0)
+    logits = torch.randn(4, 50257, generator=gen)
+    logits[0, 777] = logits[0, 40000] = 9.0
+    logits[1, 50256] = 11.0
+    logits[2, 0] = 12.0
+    dev = logits.to(DEV)
+    ids = torch.empty(4, dtype=torch.int32, device=DEV)
+    logp = torch.empty(4, dtype=torch.float32, device=DEV)
+    K.sample(dev, ids, logp)
+    want = [777, 50256, 0, int(logits[3].argmax())]
+    assert ids.tolist() == want
+    ref = torch.log_softmax(logits.double(), -1)
+    for r in range(4):
+        assert abs(float(logp[r]) - float(ref[r, want[r]])) < 1e-4
+
+
+def test_sampling_is_the_inverse_cdf_of_the_tempered_softmax():
+    import plain_gpt2 as plain
+    gen = torch.Generator().manual_seed(1)
+    rows, vocab, temperature, seed, first = 64, 517, 0.8, 1234567, 40
+    logits = torch.randn(rows, vocab, generator=gen) * 3
+    ids = torch.empty(rows, dtype=torch.int32, device=DEV)
+    logp = torch.empty(rows, dtype=torch.float32, device=DEV)
+    draw_rows = torch.arange(rows - 1, -1, -1, dtype=torch.int32, device=DEV)
+    K.sample(logits.to(DEV), ids, logp, temperature=temperature, seed=seed, first_draw=first, draw_rows=draw_rows)
+    exact = 0
+    for r in range(rows):
+        u = plain.interior_unit(plain.splitmix64(seed, first + rows - 1 - r))
+        p = torch.softmax(logits[r].double() / temperature, -1)
+        c = torch.cumsum(p, -1)
+        k = int(ids[r])
+        # the chosen index satisfies c[k-1] < u <= c[k] up to float32 rounding of the running sum
+        lo = float(c[k - 1]) if k > 0 else 0.0
+        assert lo - 1e-5 <= u <= float(c[k]) + 1e-5, (r, k, u, lo, float(c[k]))
+        exact += k == plain.sample_index(logits[r], temperature, u)
+        assert abs(float(logp[r]) - math.log(float(p[k]))) < 1e-4
+    assert exact >= rows - 2
+    # the same seed gives the same tokens; another seed does not
+    again = torch.empty_like(ids)
+    K.sample(logits.to(DEV), again, logp, temperature=temperature, seed=seed, first_draw=first, draw_rows=draw_rows)
+    assert torch.equal(ids, again)
+    K.sample(logits.to(DEV), again, logp, temperature=temperature, seed=seed + 1, first_draw=first, draw_rows=draw_rows)
+    assert not torch.equal(ids, again)

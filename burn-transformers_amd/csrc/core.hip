@@ -94,6 +94,99 @@ __global__ void add_norm_kernel(float* __restrict__ x, const float* __restrict__
   }
 }
 
+// The same for rows whose width is a multiple of four and at most 1024 * VPT (VPT up to 4): the row lives
+// in registers, every load of a thread (stream, each partial sum, bias) is independent of the
+// others and in flight at once.  A decode step has few rows, so one row's latency is what counts.
+#define ADD_NORM_MAX_SPLITS 8
+template <typename T, int VPT>
+__global__ void __launch_bounds__(256)
+add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int n_delta,
+                    int64_t delta_stride, const float* __restrict__ bias, const float* __restrict__ gamma,
+                    const float* __restrict__ beta, float eps, int kind, T* __restrict__ out,
+                    const int* __restrict__ rows, int width, int write_back) {
+  __shared__ float scratch[32];
+  const int r = blockIdx.x;
+  const int t = rows ? rows[r] : r;
+  const int quads = width >> 2;
+  float4* xr = reinterpret_cast<float4*>(x + (int64_t)t * width);
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 v[VPT], part[VPT][ADD_NORM_MAX_SPLITS], b[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    int c = threadIdx.x + i * 256;
+    bool in = c < quads;
+    v[i] = in ? xr[c] : zero;
+    b[i] = (in && bias) ? reinterpret_cast<const float4*>(bias)[c] : zero;
+#pragma unroll
+    for (int s = 0; s < ADD_NORM_MAX_SPLITS; ++s)
+      part[i][s] = (in && s < n_delta)
+                       ? reinterpret_cast<const float4*>(delta + s * delta_stride + (int64_t)t * width)[c]
+                       : zero;
+  }
+  float partial = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+#pragma unroll
+    for (int s = 0; s < ADD_NORM_MAX_SPLITS; ++s) {   // same order of additions as the plain kernel
+      v[i].x += part[i][s].x; v[i].y += part[i][s].y; v[i].z += part[i][s].z; v[i].w += part[i][s].w;
+    }
+    v[i].x += b[i].x; v[i].y += b[i].y; v[i].z += b[i].z; v[i].w += b[i].w;
+    int c = threadIdx.x + i * 256;
+    if (c < quads) {
+      if (write_back) xr[c] = v[i];
+      partial += (kind == 0) ? (v[i].x + v[i].y + v[i].z + v[i].w)
+                             : (v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w);
+    }
+  }
+  float total = block_sum(partial, scratch);
+  float mean = 0.f, rstd;
+  if (kind == 0) {
+    mean = total / (float)width;
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      if (threadIdx.x + i * 256 < quads) {
+        float a0 = v[i].x - mean, a1 = v[i].y - mean, a2 = v[i].z - mean, a3 = v[i].w - mean;
+        sq += a0 * a0 + a1 * a1 + a2 * a2 + a3 * a3;
+      }
+    }
+    float var = block_sum(sq, scratch) / (float)width;
+    rstd = 1.0f / sqrtf(var + eps);
+  } else {
+    rstd = 1.0f / sqrtf(total / (float)width + eps);
+  }
+  if (out == nullptr) return;
+  T* orow = out + (int64_t)r * width;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    int c = threadIdx.x + i * 256;
+    if (c >= quads) continue;
+    float4 g = reinterpret_cast<const float4*>(gamma)[c];
+    float4 be = beta ? reinterpret_cast<const float4*>(beta)[c] : zero;
+    float y[4] = {(v[i].x - mean) * rstd * g.x + be.x, (v[i].y - mean) * rstd * g.y + be.y,
+                  (v[i].z - mean) * rstd * g.z + be.z, (v[i].w - mean) * rstd * g.w + be.w};
+    store4<T>(orow + 4 * c, y, 4, true);
+  }
+}
+
+template <typename T>
+static void launch_add_norm(hipStream_t stream, float* x, const float* delta, int n_delta, int64_t delta_stride,
+                            const float* bias, const float* gamma, const float* beta, float eps, int kind,
+                            T* out, const int* rows, int n_rows, int width, int write_back) {
+  dim3 grid(n_rows), block(256);
+  bool vec = width % 4 == 0 && width <= 4096 && n_delta <= ADD_NORM_MAX_SPLITS && delta_stride % 4 == 0;
+#define BT_ADD_NORM_VEC(VPT)                                                                             \
+  hipLaunchKernelGGL((add_norm_vec_kernel<T, VPT>), grid, block, 0, stream, x, delta, n_delta, delta_stride, \
+                     bias, gamma, beta, eps, kind, out, rows, width, write_back)
+  if (vec && width <= 1024) BT_ADD_NORM_VEC(1);
+  else if (vec && width <= 2048) BT_ADD_NORM_VEC(2);
+  else if (vec) BT_ADD_NORM_VEC(4);
+  else
+    hipLaunchKernelGGL(add_norm_kernel<T>, grid, block, (size_t)width * sizeof(float), stream, x, delta,
+                       n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+#undef BT_ADD_NORM_VEC
+}
+
 BT_EXPORT int bt_add_norm(void* stream, int out_dtype, float* x, const float* delta, int n_delta,
                           int64_t delta_stride, const float* bias, const float* gamma,
                           const float* beta, float eps, int kind, void* out, const int* rows,
@@ -101,14 +194,12 @@ BT_EXPORT int bt_add_norm(void* stream, int out_dtype, float* x, const float* de
   if (n_rows <= 0) return BT_OK;
   if (width <= 0 || width > 15360) BT_REFUSE("add_norm: width %d outside 1..15360 (the row is held in LDS)", width);
   if (kind != 0 && kind != 1) BT_REFUSE("add_norm: unknown norm kind %d", kind);
-  dim3 grid(n_rows), block(256);
-  size_t lds = (size_t)width * sizeof(float);
   if (out_dtype == 0)
-    hipLaunchKernelGGL(add_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, x, delta, n_delta,
-                       delta_stride, bias, gamma, beta, eps, kind, (float*)out, rows, width, write_back);
+    launch_add_norm<float>((hipStream_t)stream, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind,
+                           (float*)out, rows, n_rows, width, write_back);
   else
-    hipLaunchKernelGGL(add_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, x, delta, n_delta,
-                       delta_stride, bias, gamma, beta, eps, kind, (bf16_t*)out, rows, width, write_back);
+    launch_add_norm<bf16_t>((hipStream_t)stream, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind,
+                            (bf16_t*)out, rows, n_rows, width, write_back);
   return bt_check_launch("add_norm");
 }
 

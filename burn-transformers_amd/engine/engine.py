@@ -40,7 +40,9 @@ class Engine:
         self.cache = Cache(model.kv_specs, model.state_specs, max_tokens, model.max_positions,
                            model.dtype, model.device, max_slots)
         self.pool = BufferPool(self.device)
-        self.use_graphs = graphs
+        # a mixer that plans work on the host per step cannot be replayed from a graph
+        self.use_graphs = graphs and all(getattr(block.parts.get("mixer"), "graph_safe", True)
+                                         for block in model.blocks)
         self._meta = None                  # device int32 buffer of eager steps
         self._pinned = []                  # ring of (pinned int32 tensor, event)
         self._pinned_next = 0

@@ -76,6 +76,10 @@ class Norm(Part):
 
 
 class Mixer(Part):
+    # False for a mixer whose forward reads the step's host tables (``step.host``) or otherwise
+    # does per-step work in Python: steps of a model with such a mixer are never graph-replayed
+    graph_safe = True
+
     def kv_spec(self):
         return None
 

@@ -17,8 +17,8 @@
 //   attention_prefill  one work-group per (128 queries, head, sequence); each of four waves owns
 //                      32 queries and walks the keys up to its last query's position.
 //   attention_decode   one token per sequence: one work-group per (key/value head, sequence);
-//                      the query heads sharing that head are the MFMA columns; the four waves
-//                      split the keys and meet in LDS.
+//                      the query heads sharing that head are the MFMA columns; sixteen waves
+//                      (eight for heads above 64) split the keys and meet in LDS.
 
 #include "host.h"
 #include "attention.h"
@@ -34,32 +34,53 @@ static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multip
 
 __device__ __forceinline__ bf16x8 load_bf16x8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
-// One tile of 32 keys starting at position kb (a multiple of 32) against NQ tiles of 16 queries.
-//   qpos[nq]: position of the query in column lane % 16 of tile nq, -1 if there is none.
-//   valid_end: positions >= valid_end hold no token (their values are replaced by zero).
-template <int NQ>
-__device__ __forceinline__ void attend_tile(const bf16_t* __restrict__ kplane, const bf16_t* __restrict__ vplane,
-                                            int kb, int valid_end, const int (&qpos)[NQ], int window,
-                                            float scale, const bf16x8 (&q)[NQ][NKS], floatx4 (&o)[NQ][ND],
-                                            float (&m)[NQ], float (&l)[NQ]) {
+// The operands of one tile of 32 keys, as the MFMA lanes hold them: keys for both 16-key
+// sub-tiles and every step of 32 channels, values for every block of 16 output channels.
+struct TileOperands {
+  bf16x8 k[2][NKS];
+  bf16x4 v[ND][2];
+};
+
+// Issues the loads of one tile (kb a multiple of 32); nothing waits on them here, so the caller
+// can have the next tile's loads in flight while it works on the current one.
+__device__ __forceinline__ void load_tile(TileOperands& t, const bf16_t* __restrict__ kplane,
+                                          const bf16_t* __restrict__ vplane, int kb) {
   const int lane = threadIdx.x & 63, i16 = lane & 15, g = lane >> 4;
   const int kin = kb & (BT_KV_BLOCK - 1);
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  floatx4 s[NQ][2];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    bf16x8 kop[NKS];
+  for (int h = 0; h < 2; ++h)
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       int channel = ks * 32 + g * 8;
-      kop[ks] = channel < HD ? load_bf16x8(kplane + (kin + 16 * t + i16) * HD + channel) : zero8;
+      t.k[h][ks] = channel < HD ? load_bf16x8(kplane + (kin + 16 * h + i16) * HD + channel) : zero8;
     }
+#pragma unroll
+  for (int dt = 0; dt < ND; ++dt) {
+    int channel = dt * 16 + i16;
+    t.v[dt][0] = *reinterpret_cast<const bf16x4*>(vplane + ((kin / 4 + g) * HD + channel) * 4);
+    t.v[dt][1] = *reinterpret_cast<const bf16x4*>(vplane + ((kin / 4 + 4 + g) * HD + channel) * 4);
+  }
+}
+
+// One tile of 32 keys starting at position kb against NQ tiles of 16 queries.
+//   qpos[nq]: position of the query in column lane % 16 of tile nq, -1 if there is none.
+//   valid_end: positions >= valid_end hold no token (their values are replaced by zero).
+template <int NQ>
+__device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, int valid_end,
+                                            const int (&qpos)[NQ], int window, float scale,
+                                            const bf16x8 (&q)[NQ][NKS], floatx4 (&o)[NQ][ND],
+                                            float (&m)[NQ], float (&l)[NQ]) {
+  const int lane = threadIdx.x & 63, g = lane >> 4;
+  floatx4 s[NQ][2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
 #pragma unroll
     for (int nq = 0; nq < NQ; ++nq) {
       floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[ks], q[nq][ks], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tile.k[t][ks], q[nq][ks], acc, 0, 0, 0);
       s[nq][t] = acc;
     }
   }
@@ -102,9 +123,7 @@ __device__ __forceinline__ void attend_tile(const bf16_t* __restrict__ kplane, c
   const bool ragged = kb + 32 > valid_end;
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt) {
-    int channel = dt * 16 + i16;
-    bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vplane + ((kin / 4 + g) * HD + channel) * 4);
-    bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vplane + ((kin / 4 + 4 + g) * HD + channel) * 4);
+    bf16x4 v0 = tile.v[dt][0], v1 = tile.v[dt][1];
     if (ragged) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -117,6 +136,12 @@ __device__ __forceinline__ void attend_tile(const bf16_t* __restrict__ kplane, c
     for (int nq = 0; nq < NQ; ++nq)
       o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[nq], o[nq][dt], 0, 0, 0);
   }
+}
+
+// Start of the (block, kv head) plane that holds position kb of a sequence.
+__device__ __forceinline__ int64_t tile_plane(const AttnArgs& a, int seq, int kv_head, int kb) {
+  int block = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + kb / BT_KV_BLOCK];
+  return ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
 }
 
 #define PREFILL_NQ 2
@@ -163,10 +188,18 @@ attention_prefill_kernel(AttnArgs a) {
   const int valid_end = start + count;
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
+  TileOperands current, next;
+  if (lo < hi) {
+    int64_t plane = tile_plane(a, seq, kv_head, lo);
+    load_tile(next, keys + plane, values + plane, lo);
+  }
   for (int kb = lo; kb < hi; kb += 32) {
-    int block = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + kb / BT_KV_BLOCK];
-    int64_t plane = ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
-    attend_tile<PREFILL_NQ>(keys + plane, values + plane, kb, valid_end, qpos, a.window, a.scale, q, o, m, l);
+    current = next;
+    if (kb + 32 < hi) {
+      int64_t plane = tile_plane(a, seq, kv_head, kb + 32);
+      load_tile(next, keys + plane, values + plane, kb + 32);
+    }
+    attend_tile<PREFILL_NQ>(current, kb, valid_end, qpos, a.window, a.scale, q, o, m, l);
   }
   bf16_t* out = static_cast<bf16_t*>(a.out);
 #pragma unroll
@@ -185,16 +218,19 @@ attention_prefill_kernel(AttnArgs a) {
   }
 }
 
-#define DECODE_WAVES 4
+// sixteen waves leave each lane 128 registers, eight leave 256: large heads need the latter
+#define DECODE_WAVES (HD <= 64 ? 16 : 8)
 
 __global__ void __launch_bounds__(DECODE_WAVES * 64)
 attention_decode_kernel(AttnArgs a) {
-  __shared__ float sm_m[DECODE_WAVES][16];
-  __shared__ float sm_l[DECODE_WAVES][16];
-  __shared__ float sm_o[DECODE_WAVES][16][HD];
+  // per wave: maximum and sum of each query column, and its output row; `group` columns are real
+  extern __shared__ float sm[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i16 = lane & 15, g = lane >> 4;
   const int seq = blockIdx.y, kv_head = blockIdx.x;
   const int group = a.q_heads / a.kv.kv_heads;
+  float* sm_m = sm;                                   // [DECODE_WAVES][group]
+  float* sm_l = sm + DECODE_WAVES * group;            // [DECODE_WAVES][group]
+  float* sm_o = sm + 2 * DECODE_WAVES * group;        // [DECODE_WAVES][group][HD]
   const int tok = a.seq_off[seq], pos = a.seq_start[seq];
   const bf16_t* Q = static_cast<const bf16_t*>(a.q);
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -217,36 +253,47 @@ attention_decode_kernel(AttnArgs a) {
   if (a.window > 0 && pos - a.window + 1 > 0) lo = (pos - a.window + 1) & ~31;
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
-  for (int kb = lo + 32 * wave; kb <= pos; kb += 32 * DECODE_WAVES) {
-    int block = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + kb / BT_KV_BLOCK];
-    int64_t plane = ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
-    attend_tile<1>(keys + plane, values + plane, kb, pos + 1, qpos, a.window, a.scale, q, o, m, l);
+  const int first = lo + 32 * wave, stride = 32 * DECODE_WAVES;
+  TileOperands current, next;
+  if (first <= pos) {
+    int64_t plane = tile_plane(a, seq, kv_head, first);
+    load_tile(next, keys + plane, values + plane, first);
+  }
+  for (int kb = first; kb <= pos; kb += stride) {
+    current = next;
+    if (kb + stride <= pos) {
+      int64_t plane = tile_plane(a, seq, kv_head, kb + stride);
+      load_tile(next, keys + plane, values + plane, kb + stride);
+    }
+    attend_tile<1>(current, kb, pos + 1, qpos, a.window, a.scale, q, o, m, l);
   }
   float total = l[0];
   total += __shfl_xor(total, 16, 64);
   total += __shfl_xor(total, 32, 64);
-  if (g == 0) {
-    sm_m[wave][i16] = m[0];
-    sm_l[wave][i16] = total;
+  if (has_query) {
+    if (g == 0) {
+      sm_m[wave * group + i16] = m[0];
+      sm_l[wave * group + i16] = total;
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sm_o[(wave * group + i16) * HD + dt * 16 + 4 * g + r] = o[0][dt][r];
   }
-#pragma unroll
-  for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) sm_o[wave][i16][dt * 16 + 4 * g + r] = o[0][dt][r];
   __syncthreads();
   bf16_t* out = static_cast<bf16_t*>(a.out);
   for (int e = threadIdx.x; e < group * HD; e += DECODE_WAVES * 64) {
     int j = e / HD, channel = e % HD;
-    float top = sm_m[0][j];
+    float top = sm_m[j];
 #pragma unroll
-    for (int w = 1; w < DECODE_WAVES; ++w) top = fmaxf(top, sm_m[w][j]);
+    for (int w = 1; w < DECODE_WAVES; ++w) top = fmaxf(top, sm_m[w * group + j]);
     float num = 0.f, den = 0.f;
     if (top != -INFINITY) {
 #pragma unroll
       for (int w = 0; w < DECODE_WAVES; ++w) {
-        float f = __expf(sm_m[w][j] - top);
-        num += sm_o[w][j][channel] * f;
-        den += sm_l[w][j] * f;
+        float f = __expf(sm_m[w * group + j] - top);
+        num += sm_o[(w * group + j) * HD + channel] * f;
+        den += sm_l[w * group + j] * f;
       }
     }
     out[(int64_t)tok * a.ldo + (kv_head * group + j) * HD + channel] = (bf16_t)(den > 0.f ? num / den : 0.f);
@@ -286,6 +333,8 @@ BT_EXPORT int bt_attention_decode_bf16(void* stream, const AttnArgs* args) {
               args->q_heads / args->kv.kv_heads);
   if (args->n_tokens != args->n_seqs) BT_REFUSE("attention_decode_bf16: needs exactly one token per sequence");
   dim3 grid(args->kv.kv_heads, args->n_seqs);
-  hipLaunchKernelGGL(attention_decode_kernel, grid, dim3(DECODE_WAVES * 64), 0, (hipStream_t)stream, *args);
+  int group = args->q_heads / args->kv.kv_heads;
+  size_t lds = (size_t)DECODE_WAVES * group * (HD + 2) * sizeof(float);
+  hipLaunchKernelGGL(attention_decode_kernel, grid, dim3(DECODE_WAVES * 64), lds, (hipStream_t)stream, *args);
   return bt_check_launch("attention_decode_bf16");
 }

@@ -434,7 +434,7 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t seed, uint64_t index) {
   return v ^ (v >> 31);
 }
 
-#define SAMPLE_THREADS 256
+#define SAMPLE_THREADS 1024
 
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int sample, float temperature,
@@ -450,7 +450,7 @@ sample_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int sampl
   // the logits are divided by the temperature only when sampling
   float divisor = sample ? temperature : 1.0f;
 
-  // maximum and its lowest index
+  // maximum and its lowest index; a thread sees its indices in rising order, so `>` keeps the lowest
   float top = -INFINITY;
   int arg = 0x7fffffff;
   for (int k = tid; k < vocab; k += SAMPLE_THREADS) {
@@ -469,6 +469,17 @@ sample_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int sampl
     if (best_value[w] > top || (best_value[w] == top && best_index[w] < arg)) { top = best_value[w]; arg = best_index[w]; }
   }
 
+  if (!sample) {
+    float mine = 0.f;
+    for (int k = tid; k < vocab; k += SAMPLE_THREADS) mine += expf(z[k] - top);
+    float total = block_sum(mine, scratch);
+    if (tid == 0) {
+      ids[row] = arg;
+      logp[row] = z[arg] - top - logf(total);
+    }
+    return;
+  }
+
   // each thread owns one contiguous segment of the vocabulary, so that prefix sums run in index order
   int seg = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
   int lo = tid * seg, hi = lo + seg < vocab ? lo + seg : vocab;
@@ -476,36 +487,31 @@ sample_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int sampl
   for (int k = lo; k < hi; ++k) mine += expf(z[k] / divisor - top);
   seg_sum[tid] = mine;
   float total = block_sum(mine, scratch);  // also orders the seg_sum writes before the reads below
-
-  int pick = arg;
-  if (sample) {
-    if (tid == 0) {
-      float u = (float)(((double)(splitmix64(seed, first_draw + (uint64_t)(draw_rows ? draw_rows[row] : row)) >> 41) + 0.5) / 8388608.0);
-      float running = 0.f;
-      for (int t = 0; t < SAMPLE_THREADS; ++t) running += seg_sum[t];   // realised total in index order
-      float threshold = u * running;
-      float before = 0.f;
-      int owner = SAMPLE_THREADS - 1;
-      for (int t = 0; t < SAMPLE_THREADS; ++t) {
-        if (before + seg_sum[t] >= threshold) { owner = t; break; }
-        before += seg_sum[t];
-      }
-      int olo = owner * seg, ohi = olo + seg < vocab ? olo + seg : vocab;
-      int k = olo;
-      float c = before;
-      for (; k < ohi; ++k) {
-        c += expf(z[k] / divisor - top);
-        if (!(c < threshold)) break;
-      }
-      if (k >= vocab) k = vocab - 1;
-      chosen = k;
-    }
-    __syncthreads();
-    pick = chosen;
-  }
   if (tid == 0) {
-    ids[row] = pick;
-    logp[row] = z[pick] / divisor - top - logf(total);
+    float u = (float)(((double)(splitmix64(seed, first_draw + (uint64_t)(draw_rows ? draw_rows[row] : row)) >> 41) + 0.5) / 8388608.0);
+    float running = 0.f;
+    for (int t = 0; t < SAMPLE_THREADS; ++t) running += seg_sum[t];   // realised total in index order
+    float threshold = u * running;
+    float before = 0.f;
+    int owner = SAMPLE_THREADS - 1;
+    for (int t = 0; t < SAMPLE_THREADS; ++t) {
+      if (before + seg_sum[t] >= threshold) { owner = t; break; }
+      before += seg_sum[t];
+    }
+    int olo = owner * seg, ohi = olo + seg < vocab ? olo + seg : vocab;
+    int k = olo;
+    float c = before;
+    for (; k < ohi; ++k) {
+      c += expf(z[k] / divisor - top);
+      if (!(c < threshold)) break;
+    }
+    if (k >= vocab) k = vocab - 1;
+    chosen = k;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    ids[row] = chosen;
+    logp[row] = z[chosen] / divisor - top - logf(total);
   }
 }
 

@@ -110,19 +110,21 @@ add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int 
   const int quads = width >> 2;
   float4* xr = reinterpret_cast<float4*>(x + (int64_t)t * width);
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-  float4 v[VPT], part[VPT][ADD_NORM_MAX_SPLITS], b[VPT];
+  float4 v[VPT], part[VPT][ADD_NORM_MAX_SPLITS], b[VPT], g[VPT], be[VPT];
+  // every load of the kernel is issued here, before anything waits: one trip to memory
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     int c = threadIdx.x + i * 256;
-    bool in = c < quads;
-    v[i] = in ? xr[c] : zero;
-    b[i] = (in && bias) ? reinterpret_cast<const float4*>(bias)[c] : zero;
+    int cc = c < quads ? c : 0;
+    v[i] = xr[cc];
+    b[i] = bias ? reinterpret_cast<const float4*>(bias)[cc] : zero;
+    g[i] = (out != nullptr) ? reinterpret_cast<const float4*>(gamma)[cc] : zero;
+    be[i] = (out != nullptr && beta) ? reinterpret_cast<const float4*>(beta)[cc] : zero;
 #pragma unroll
     for (int s = 0; s < ADD_NORM_MAX_SPLITS; ++s)
-      part[i][s] = (in && s < n_delta)
-                       ? reinterpret_cast<const float4*>(delta + s * delta_stride + (int64_t)t * width)[c]
-                       : zero;
-  }
+      part[i][s] = (s < n_delta) ? reinterpret_cast<const float4*>(delta + s * delta_stride + (int64_t)t * width)[cc]
+                                 : zero;
+  }   // lanes beyond the row read column 0; whatever they hold is never used below
   float partial = 0.f;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
@@ -161,10 +163,8 @@ add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int 
   for (int i = 0; i < VPT; ++i) {
     int c = threadIdx.x + i * 256;
     if (c >= quads) continue;
-    float4 g = reinterpret_cast<const float4*>(gamma)[c];
-    float4 be = beta ? reinterpret_cast<const float4*>(beta)[c] : zero;
-    float y[4] = {(v[i].x - mean) * rstd * g.x + be.x, (v[i].y - mean) * rstd * g.y + be.y,
-                  (v[i].z - mean) * rstd * g.z + be.z, (v[i].w - mean) * rstd * g.w + be.w};
+    float y[4] = {(v[i].x - mean) * rstd * g[i].x + be[i].x, (v[i].y - mean) * rstd * g[i].y + be[i].y,
+                  (v[i].z - mean) * rstd * g[i].z + be[i].z, (v[i].w - mean) * rstd * g[i].w + be[i].w};
     store4<T>(orow + 4 * c, y, 4, true);
   }
 }
@@ -254,7 +254,7 @@ gemm_plain_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W,
 }
 
 int bt_check_epilogue(const Epilogue& e, int N, const char* who) {
-  if (e.mode < 0 || e.mode > 3) BT_REFUSE("%s: unknown epilogue mode %d", who, e.mode);
+  if (e.mode < 0 || e.mode > 4) BT_REFUSE("%s: unknown epilogue mode %d", who, e.mode);
   if (e.out == nullptr) BT_REFUSE("%s: epilogue has no output", who);
   if (e.mode == EPI_QKV) {
     if (e.kv.head_dim <= 0 || e.kv.head_dim % 16 != 0)

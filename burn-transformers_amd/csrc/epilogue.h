@@ -11,6 +11,7 @@ enum EpilogueMode {
   EPI_ACT = 1,    // out[m][n] = act(acc + bias)                 (element type T)
   EPI_F32 = 2,    // out[split][m][n] = acc (+ bias in split 0)  (float; the consumer sums the splits)
   EPI_QKV = 3,    // columns [0,n_q) -> out, [n_q,n_q+n_kv) -> keys, the next n_kv -> values
+  EPI_RESIDUAL = 4,  // out[m][n] += acc + bias                  (float: the residual stream itself)
 };
 
 enum Activation {
@@ -51,7 +52,9 @@ __device__ __forceinline__ void store4<float>(float* dst, const float* v, int co
   if (count == 4 && aligned) {
     *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
   } else {
-    for (int i = 0; i < count; ++i) dst[i] = v[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < count) dst[i] = v[i];
   }
 }
 template <>
@@ -60,7 +63,99 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const float* v, int 
     bf16x4 packed = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
     *reinterpret_cast<bf16x4*>(dst) = packed;
   } else {
-    for (int i = 0; i < count; ++i) dst[i] = (bf16_t)v[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < count) dst[i] = (bf16_t)v[i];
+  }
+}
+
+// What an epilogue needs from memory besides the accumulators, fetched at the START of a kernel
+// so that no load is left on the critical path after the last multiply: the bias (plus the old
+// value of the residual stream in EPI_RESIDUAL) and, for the key/value scatter, where the row's
+// token lives in the paged cache.
+struct EpiloguePrefetch {
+  float add[4];
+  int64_t kv_base;   // start of the (block, head) plane of the token; valid for key/value columns
+  int pos;
+};
+
+// A valid address for the loads of an epilogue mode that is not in use: the prefetch below has
+// no branches, so every load in it is always issued (and its result discarded where unused).
+__device__ int bt_dummy_words[4] = {0, 0, 0, 0};
+
+__device__ __forceinline__ EpiloguePrefetch epilogue_prefetch(const Epilogue& e, int M, int N, int m, int n0,
+                                                              int split) {
+  // Branch-free on purpose: with no control flow the compiler issues these loads among the
+  // caller's own and waits for none of them before it has to.
+  EpiloguePrefetch p;
+  const int mm = m < M ? m : M - 1;
+  const bool with_bias = e.bias != nullptr && split == 0;
+  const bool residual = e.mode == EPI_RESIDUAL;
+  const bool scatter = e.mode == EPI_QKV;
+  const float* dummy = reinterpret_cast<const float*>(bt_dummy_words);
+  const float* bias = with_bias ? e.bias : dummy;
+  const float* x = residual ? static_cast<const float*>(e.out) + (int64_t)mm * e.ldo : dummy;
+  const int* tok_seq = scatter ? e.tok_seq : bt_dummy_words;
+  const int* tok_pos = scatter ? e.tok_pos : bt_dummy_words;
+  int seq = tok_seq[scatter ? mm : 0];
+  int pos = tok_pos[scatter ? mm : 0];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int nn = n0 + i < N ? n0 + i : N - 1;
+    float b = bias[with_bias ? nn : 0];
+    float xv = x[residual ? nn : 0];
+    p.add[i] = (with_bias ? b : 0.f) + (residual ? xv : 0.f);
+  }
+  // key/value columns: where the token's position lives in the paged cache
+  int c = n0 - e.n_q;
+  if (c >= e.n_kv) c -= e.n_kv;
+  const bool kv_column = scatter && n0 >= e.n_q && n0 < N;
+  const int head = kv_column ? c / e.kv.head_dim : 0;
+  const int* blocks = kv_column ? e.kv.blocks : bt_dummy_words;
+  int block = blocks[kv_column ? (int64_t)seq * e.kv.max_blocks + pos / BT_KV_BLOCK : 0];
+  p.kv_base = ((int64_t)block * e.kv.kv_heads + head) * (int64_t)(BT_KV_BLOCK * e.kv.head_dim);
+  p.pos = pos;
+  return p;
+}
+
+// The epilogue with everything but the accumulators already in registers.
+template <typename T>
+__device__ __forceinline__ void epilogue4_prefetched(const Epilogue& e, int N, int m, int n0, const float* acc,
+                                                     int split, const EpiloguePrefetch& p) {
+  int count = N - n0 < 4 ? N - n0 : 4;
+  if (count <= 0) return;
+  float v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = acc[i] + p.add[i];
+  bool aligned = (e.ldo & 3) == 0;
+  if (e.mode == EPI_STORE) {
+    store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+  } else if (e.mode == EPI_ACT) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = activate(v[i], e.act);
+    store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+  } else if (e.mode == EPI_F32) {
+    store4<float>(static_cast<float*>(e.out) + (int64_t)split * e.split_stride + (int64_t)m * e.ldo + n0,
+                  v, count, aligned);
+  } else if (e.mode == EPI_RESIDUAL) {
+    store4<float>(static_cast<float*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+  } else {
+    if (n0 < e.n_q) {
+      store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+    } else {
+      int c = n0 - e.n_q;
+      bool is_value = c >= e.n_kv;
+      if (is_value) c -= e.n_kv;
+      int channel = c % e.kv.head_dim;
+      if (!is_value) {
+        store4<T>(static_cast<T*>(e.kv.keys) + p.kv_base + key_offset(e.kv.head_dim, p.pos, channel), v, count, true);
+      } else {
+        T* dst = static_cast<T*>(e.kv.values) + p.kv_base + value_offset(e.kv.head_dim, p.pos, channel);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)     // consecutive channels of one position lie four elements apart
+          if (i < count) dst[4 * i] = from_float<T>(v[i]);
+      }
+    }
   }
 }
 
@@ -87,6 +182,12 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int N, int m, int n
   } else if (e.mode == EPI_F32) {
     store4<float>(static_cast<float*>(e.out) + (int64_t)split * e.split_stride + (int64_t)m * e.ldo + n0,
                   v, count, aligned);
+  } else if (e.mode == EPI_RESIDUAL) {
+    float* x = static_cast<float*>(e.out) + (int64_t)m * e.ldo + n0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < count) v[i] += x[i];
+    store4<float>(x, v, count, aligned);
   } else {  // EPI_QKV: n_q, n_kv and head_dim are multiples of 16, so the four columns share a head
     if (n0 < e.n_q) {
       store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
@@ -101,8 +202,10 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int N, int m, int n
         store4<T>(static_cast<T*>(e.kv.keys) + base + key_offset(e.kv.head_dim, pos, channel), v, count,
                   true);
       } else {
-        T* dst = static_cast<T*>(e.kv.values) + base;
-        for (int i = 0; i < count; ++i) dst[value_offset(e.kv.head_dim, pos, channel + i)] = from_float<T>(v[i]);
+        T* dst = static_cast<T*>(e.kv.values) + base + value_offset(e.kv.head_dim, pos, channel);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)     // consecutive channels of one position lie four elements apart
+          if (i < count) dst[4 * i] = from_float<T>(v[i]);
       }
     }
   }

@@ -23,6 +23,8 @@
 #define TILE_K 64
 #define TILE_ROW_BYTES 128
 
+__device__ __forceinline__ int chunks_of(int K) { return (K + 31) / 32; }
+
 __device__ __forceinline__ int swizzled(int row, int chunk) {
   return row * TILE_ROW_BYTES + ((chunk ^ (row & 7)) << 4);
 }
@@ -124,66 +126,94 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
   }
 }
 
-#define SKINNY_WAVES 8
-
-template <int MT, int U>
-__global__ void __launch_bounds__(SKINNY_WAVES * 64)
+// Memory latency on this GPU is about a microsecond and one compute unit alone pulls only a few
+// per cent of the HBM bandwidth, while a decode step is hundreds of short kernels.  So the
+// skinny kernel (a) wants at least as many work-groups as there are compute units, which is
+// what splitting K is for when there are few output columns, and (b) has ONE round trip to
+// memory on its critical path: everything the epilogue needs (bias, old residual, cache
+// addresses) is fetched together with the first batch of weights, without a branch in between.
+template <int MT, int U, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
                    int K, Epilogue epi) {
-  __shared__ __attribute__((aligned(16))) float red[SKINNY_WAVES][MT][64][4];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  __shared__ __attribute__((aligned(16))) float red[WAVES][MT][64][4];
+  // the wave's number is the same in all its lanes: saying so keeps every test on it a scalar
+  // branch, which costs no wait for loads in flight (a divergent one does)
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int i16 = lane & 15, g = lane >> 4;
   const int n_base = blockIdx.x * 16;
   const int split = blockIdx.y, splits = gridDim.y;
   int n = n_base + i16;
   n = n < N ? n : N - 1;
-  const bf16_t* w_src = W + (int64_t)n * K + g * 8;
-  const bf16_t* a_src[MT];
-  bool a_ok[MT];
+  const bf16_t* w_row = W + (int64_t)n * K;
+  const bf16_t* a_row[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     int m = mt * 16 + i16;
-    a_ok[mt] = m < M;
-    a_src[mt] = A + (int64_t)(m < M ? m : M - 1) * lda + g * 8;
+    a_row[mt] = A + (int64_t)(m < M ? m : M - 1) * lda;
   }
+  // A batch is two phases.  First every load of the batch is issued: a chunk of 32 beyond K is
+  // skipped by a scalar branch, a group of eight beyond K (a multiple of 8) inside the last chunk
+  // reads the row's last group instead.  Only then are the weights of such a group cleared (with
+  // a bit mask) and multiplied.  Nothing that depends on a lane or on loaded data stands between
+  // the loads, so the compiler has no reason to wait for one before it issues the next.
+  // Rows beyond M repeat row M - 1; their results are dropped by the epilogue.
+  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
+  const int chunks = chunks_of(K);
+  const int stride = splits * WAVES;
   floatx4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  const int stride = splits * SKINNY_WAVES;
-  const int chunks = (K + 31) / 32;
-  for (int c0 = split * SKINNY_WAVES + wave; c0 < chunks; c0 += stride * U) {
-    bf16x8 wv[U], av[U][MT];
+  int4v wv[U], av[U][MT];
+  auto issue = [&](int c0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int cc = c0 + u * stride;
-      bool inside = cc * 32 + g * 8 < K;   // K is a multiple of 8: a group of eight is in or out
-      wv[u] = inside ? *reinterpret_cast<const bf16x8*>(w_src + (int64_t)cc * 32) : zero;
+      wv[u] = int4v{0, 0, 0, 0};
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        av[u][mt] = (inside && a_ok[mt]) ? *reinterpret_cast<const bf16x8*>(a_src[mt] + (int64_t)cc * 32) : zero;
+      for (int mt = 0; mt < MT; ++mt) av[u][mt] = int4v{0, 0, 0, 0};
+      if (cc < chunks) {
+        int k = cc * 32 + g * 8;
+        int kc = k < K ? k : K - 8;
+        wv[u] = *reinterpret_cast<const int4v*>(w_row + kc);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + kc);
+      }
     }
+  };
+  auto multiply = [&](int c0) {
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+      int keep = (c0 + u * stride) * 32 + g * 8 < K ? -1 : 0;
+      bf16x8 w = __builtin_bit_cast(bf16x8, wv[u] & keep);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u], av[u][mt], acc[mt], 0, 0, 0);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, __builtin_bit_cast(bf16x8, av[u][mt]), acc[mt], 0, 0, 0);
+    }
+  };
+  int c0 = split * WAVES + wave;
+  issue(c0);
+  // wave w < MT finishes row block w: lane holds D[i][j], i = 4 * (lane / 16) + r (column n),
+  // j = lane % 16 (row m); what its epilogue needs is fetched now, behind the first batch
+  const int out_m = (wave < MT ? wave : 0) * 16 + i16, out_n0 = n_base + g * 4;
+  EpiloguePrefetch pre = {};
+  if (wave < MT) pre = epilogue_prefetch(epi, M, N, out_m, out_n0, split);
+  multiply(c0);
+  for (c0 += stride * U; c0 < chunks; c0 += stride * U) {
+    issue(c0);
+    multiply(c0);
   }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
     *reinterpret_cast<floatx4*>(&red[wave][mt][lane][0]) = acc[mt];
   __syncthreads();
-  // wave w adds up the eight partial sums of row block w; lane holds D[i][j] with
-  // i = 4 * (lane / 16) + r (column n), j = lane % 16 (row m)
   if (wave < MT) {
     float v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < SKINNY_WAVES; ++w)
+    for (int w = 0; w < WAVES; ++w)
 #pragma unroll
       for (int r = 0; r < 4; ++r) v[r] += red[w][wave][lane][r];
-    int m = wave * 16 + i16;
-    if (m < M) epilogue4<bf16_t>(epi, N, m, n_base + g * 4, v, split);
+    if (out_m < M) epilogue4_prefetched<bf16_t>(epi, N, out_m, out_n0, v, split, pre);
   }
 }
 
@@ -193,7 +223,7 @@ static int check_operands(const char* who, const void* A, int64_t lda, const voi
   if (K % 8 != 0 || lda % 8 != 0)
     BT_REFUSE("%s: K %d and the row pitch %lld must be multiples of 8 (16-byte loads)", who, K, (long long)lda);
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) BT_REFUSE("%s: operands must be 16-byte aligned", who);
-  if (e.mode < 0 || e.mode > 3 || e.out == nullptr) BT_REFUSE("%s: bad epilogue", who);
+  if (e.mode < 0 || e.mode > 4 || e.out == nullptr) BT_REFUSE("%s: bad epilogue", who);
   if (splits < 1 || (splits > 1 && e.mode != EPI_F32))
     BT_REFUSE("%s: K can be split %d ways only into 32-bit partial sums", who, splits);
   if (e.mode == EPI_QKV) {
@@ -225,15 +255,15 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
   if (M > 64) BT_REFUSE("gemm_skinny_bf16: %d rows, at most 64", M);
   int rc = check_operands("gemm_skinny_bf16", A, lda, W, M, N, K, *epi, splits);
   if (rc) return rc;
-  dim3 grid((N + 15) / 16, splits), block(SKINNY_WAVES * 64);
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
+  dim3 grid((N + 15) / 16, splits);
   if (M <= 16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, 8>), grid, block, 0, s, a, lda, w, M, N, K, *epi);
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, 8, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi);
   else if (M <= 32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 4>), grid, block, 0, s, a, lda, w, M, N, K, *epi);
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, 4, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi);
   else
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2>), grid, block, 0, s, a, lda, w, M, N, K, *epi);
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi);
   return bt_check_launch("gemm_skinny_bf16");
 }

@@ -15,7 +15,7 @@ from . import build
 FLOAT32, BFLOAT16 = 0, 1
 DTYPE_CODES = {torch.float32: FLOAT32, torch.bfloat16: BFLOAT16}
 
-EPI_STORE, EPI_ACT, EPI_F32, EPI_QKV = 0, 1, 2, 3
+EPI_STORE, EPI_ACT, EPI_F32, EPI_QKV, EPI_RESIDUAL = 0, 1, 2, 3, 4
 ACTIVATIONS = {"gelu_tanh": 0, "gelu_erf": 1}
 NORM_KINDS = {"layer_norm": 0, "rms_norm": 1}
 KV_BLOCK = 64
@@ -113,6 +113,11 @@ def epilogue_f32(out, bias=None):
     split_stride = out.stride(0) if out.dim() == 3 else 0
     return Epilogue(mode=EPI_F32, bias=_ptr(bias), out=out.data_ptr(), ldo=out.stride(-2),
                     split_stride=split_stride)
+
+
+def epilogue_residual(x, bias=None):
+    """x[m][n] += acc + bias, with x the float32 residual stream [M, N] itself."""
+    return Epilogue(mode=EPI_RESIDUAL, bias=_ptr(bias), out=x.data_ptr(), ldo=x.stride(0))
 
 
 def epilogue_qkv(q_out, n_q, n_kv, kv_view, tok_seq, tok_pos, bias=None):

@@ -3,5 +3,5 @@ from .base import (Block, Delta, Embedding, FeedForward, Memory, Mixer, Norm, Pa
                    ResidualStream)
 from .registry import lookup, register, unregister
 
-__all__ = ["Block", "Delta", "Embedding", "FeedForward", "Memory", "Mixer", "Norm", "Part", "Readout",
-           "ResidualStream", "lookup", "register", "unregister"]
+__all__ = ["Block", "Delta", "Embedding", "FeedForward", "Memory", "Mixer", "Norm", "Part",
+           "Readout", "ResidualStream", "lookup", "register", "unregister"]

@@ -8,7 +8,7 @@ heads*head_dim] with its bias.
 One step: the fused projection's epilogue writes the queries to a buffer and scatters the new
 keys and values straight into the cache at each token's position; the attention kernel then
 reads the cache (prefill: tiled, online softmax; decode: one query per head, keys split over
-the waves); the output projection leaves 32-bit partial sums for the next norm to add.
+the waves); the output projection adds into the residual stream.
 Formulas: src/attention.rs:481-513 (projections), src/attention/dispatch.rs:314-328, 365-367,
 390-406 (scaled scores, exclusion by -inf, 32-bit softmax), src/attention.rs:882-897 (merge and
 output projection).
@@ -16,7 +16,7 @@ output projection).
 
 from ..cache.storage import KVSpec
 from ..kernels import library as K
-from .base import Delta, Mixer, split_count
+from .base import Mixer
 from .registry import register
 
 
@@ -49,7 +49,7 @@ class CausalSelfAttention(Mixer):
     def head_dims(self):
         return (self.head_dim,)
 
-    def forward(self, h, step, memory):
+    def forward(self, h, step, memory, stream):
         tokens = h.shape[0]
         kv = memory.kv()
         q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
@@ -63,8 +63,4 @@ class CausalSelfAttention(Mixer):
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                 self.heads, step.n_seqs, step.max_count, self.scale, self.window)
         K.attention(args, step.dtype, step.decode)
-        splits = split_count(tokens, self.width, self.n_q) if step.dtype_is_bf16 else 1
-        partials = step.buffer("attention.delta", splits * tokens, self.width, "float32").view(
-            splits, tokens, self.width)
-        K.gemm(mixed, self.out_weight, K.epilogue_f32(partials), splits=splits)
-        return Delta(partials, self.out_bias)
+        stream.add_product(step, mixed, self.out_weight, self.out_bias)

@@ -11,10 +11,11 @@
 No part knows which model it is in: it gets its sizes and constants as parameters and its
 tensors by role from the weight store.
 
-The residual stream is kept in float32 in both precisions, and a part's contribution is not
-added at once: it is left as a :class:`Delta` (32-bit partial sums of a matrix product, plus a
-bias) that the next norm adds while it reads the stream anyway.  That saves one pass over the
-stream per part and lets a matrix product split its K range without a reduction pass.
+The residual stream is kept in float32 in both precisions.  A part adds to it in one of two
+ways: ``stream.add_product(step, a, weight, bias)`` lets the matrix product's epilogue add into
+the stream directly (or, where splitting K pays, leaves 32-bit partial sums pending), and
+``stream.add(Delta)`` leaves any float32 tensor pending; what is pending is added by the next
+norm while it reads the stream anyway.
 """
 
 from dataclasses import dataclass
@@ -42,6 +43,21 @@ class ResidualStream:
         if self.pending is not None:
             self.flush()
         self.pending = delta
+
+    def add_product(self, step, a, weight, bias=None):
+        """x += a . weight^T + bias.  With bfloat16 and up to 64 rows (decode) the product splits its K
+        range into partial sums that stay pending: a weight-streaming product with few output columns
+        needs the extra work-groups to pull its matrix through HBM.  Otherwise the product's epilogue
+        adds into the stream in place."""
+        rows, width = a.shape[0], weight.shape[0]
+        splits = split_count(rows, width, a.shape[1]) if step.dtype_is_bf16 else 1
+        if splits > 1:
+            partials = step.buffer("stream.partials", splits * rows, width, "float32").view(splits, rows, width)
+            K.gemm(a, weight, K.epilogue_f32(partials), splits=splits)
+            self.add(Delta(partials, bias))
+        else:
+            self.flush()
+            K.gemm(a, weight, K.epilogue_residual(self.x, bias))
 
     def flush(self):
         """Adds what is pending without normalising anything."""
@@ -72,6 +88,7 @@ class Part:
 
 class Norm(Part):
     def apply(self, stream, step, rows=None):
+        """Normalised rows as a tensor [rows, width] in the step's dtype."""
         raise NotImplementedError
 
 
@@ -90,12 +107,14 @@ class Mixer(Part):
         """Head sizes for which attention kernels must be built."""
         return ()
 
-    def forward(self, h, step, memory):
+    def forward(self, h, step, memory, stream):
+        """Adds the mixer's contribution to ``stream`` (or returns it as a Delta)."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, h, step):
+    def forward(self, h, step, stream):
+        """Adds the feed-forward's contribution to ``stream`` (or returns it as a Delta)."""
         raise NotImplementedError
 
 
@@ -124,6 +143,8 @@ def split_count(rows, columns, k):
         return 1
     tiles = (columns + 15) // 16
     splits = 1
-    while tiles * splits < 512 and splits < 8 and k // (splits * 2) >= 256:
+    # at least as many work-groups as compute units (256), and still a few chunks of 32 for
+    # each of a work-group's eight waves
+    while tiles * splits < 384 and splits < 8 and k // (splits * 2) >= 400:
         splits *= 2
     return splits

@@ -1,8 +1,8 @@
 """Arrangements of parts in a layer.
 
 pre_norm: y = x + mixer(norm(x)); z = y + feed_forward(norm(y))
-(src/models/gpt2/model.rs:218-270).  Each contribution is left pending on the stream and
-added by the norm that reads the stream next.
+(src/models/gpt2/model.rs:218-270).  A part adds its contribution to the stream itself or
+returns it as a Delta, which stays pending until the next norm reads the stream.
 """
 
 from .base import Block
@@ -15,5 +15,10 @@ class PreNormBlock(Block):
 
     def forward(self, stream, step, memory):
         parts = self.parts
-        stream.add(parts["mixer"].forward(parts["mixer_norm"].apply(stream, step), step, memory))
-        stream.add(parts["ff"].forward(parts["ff_norm"].apply(stream, step), step))
+        mixer, ff = parts["mixer"], parts["ff"]
+        delta = mixer.forward(parts["mixer_norm"].apply(stream, step), step, memory, stream)
+        if delta is not None:
+            stream.add(delta)
+        delta = ff.forward(parts["ff_norm"].apply(stream, step), step, stream)
+        if delta is not None:
+            stream.add(delta)

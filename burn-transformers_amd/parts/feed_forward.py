@@ -3,11 +3,11 @@
 Parameters: width, inner, activation ("gelu_tanh": 0.5x(1+tanh(sqrt(2/pi)(x+0.044715x^3))),
 "gelu_erf": x(1+erf(x/sqrt 2))/2; src/feed_forward.rs:351-387).  The activation runs in 32-bit
 inside the up projection's epilogue (src/feed_forward.rs:397-406 widens half inputs too); the
-down projection leaves 32-bit partial sums for the next norm to add.
+down projection adds into the residual stream.
 """
 
 from ..kernels import library as K
-from .base import Delta, FeedForward, split_count
+from .base import FeedForward
 from .registry import register
 
 
@@ -26,12 +26,8 @@ class DenseFeedForward(FeedForward):
                              f"{tuple(self.down_weight.shape)}, expected {(self.inner, self.width)} and "
                              f"{(self.width, self.inner)}")
 
-    def forward(self, h, step):
+    def forward(self, h, step, stream):
         tokens = h.shape[0]
         hidden = step.buffer("feed_forward.hidden", tokens, self.inner, step.dtype)
         K.gemm(h, self.up_weight, K.epilogue_act(hidden, self.activation, self.up_bias))
-        splits = split_count(tokens, self.width, self.inner) if step.dtype_is_bf16 else 1
-        partials = step.buffer("feed_forward.delta", splits * tokens, self.width, "float32").view(
-            splits, tokens, self.width)
-        K.gemm(hidden, self.down_weight, K.epilogue_f32(partials), splits=splits)
-        return Delta(partials, self.down_bias)
+        stream.add_product(step, hidden, self.down_weight, self.down_bias)

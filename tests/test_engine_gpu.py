@@ -134,6 +134,25 @@ def test_unequal_batches_one_after_another(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,count", [("A", 16), ("B", 17), ("A", 40), ("B", 64)])
+def test_wide_decode_batches(name, dtype, count):
+    """Decode steps of 16, 17..64 sequences take other kernels than small batches do."""
+    engine = engine_for(name, dtype, max_tokens=64 * count)
+    lengths = [3 + (7 * i) % 20 for i in range(count)]
+    requests = prompts_for(name, [n + 3 for n in lengths], seed=70)
+    slots = [engine.open() for _ in requests]
+    for begin in range(0, count, 8):
+        part = range(begin, min(begin + 8, count))
+        engine.step([(slots[i], requests[i][:lengths[i]]) for i in part], want=[[] for _ in part])
+    got = []
+    for t in range(3):
+        got.append(engine.step([(s, [r[n + t]]) for s, r, n in zip(slots, requests, lengths)]).clone())
+    for i in (0, 1, count // 2, count - 1):
+        want = plain_logits(name, requests[i])[lengths[i]:]
+        check(torch.stack([g[i] for g in got]), want, dtype, f"{name} sequence {i} of {count}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_reused_blocks_do_not_leak(dtype):
     """A slot's blocks are poisoned with NaN after it is closed; the next occupant must not care."""
     engine = engine_for("A", dtype, max_tokens=256)

@@ -64,6 +64,18 @@ def test_gemm_split_k_partials(impl, m, n, k, splits):
     assert rel_err(parts.sum(0), want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
 
 
+@pytest.mark.parametrize("impl,dtype,m,n,k", [("plain", "float32", 9, 50, 24), ("tile", "bfloat16", 130, 96, 200),
+                                               ("skinny", "bfloat16", 8, 1600, 6400), ("skinny", "bfloat16", 3, 40, 96)])
+def test_gemm_adds_into_the_residual_stream(impl, dtype, m, n, k):
+    a, w, bias, want = operands(m, n, k, DTYPES[dtype], seed=77)
+    gen = torch.Generator().manual_seed(1)
+    x0 = torch.randn(m, n, generator=gen)
+    x = x0.clone().to(DEV)
+    K.gemm(a, w, K.epilogue_residual(x, bias), impl=impl)
+    tol = 2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k)
+    assert rel_err(x, x0.double() + want + bias.cpu().double()) < tol
+
+
 def test_gemm_refuses_what_it_cannot_take():
     a, w, bias, _ = operands(4, 32, 20, torch.bfloat16)
     out = torch.empty(4, 32, dtype=torch.bfloat16, device=DEV)

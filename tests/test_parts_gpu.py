@@ -70,11 +70,13 @@ def test_dense_feed_forward_alone(dtype, width, inner, activation, tokens):
         {"width": width, "inner": inner, "activation": activation},
         {"up_weight": up.to(DEV), "up_bias": up_b.to(DEV), "down_weight": down.to(DEV), "down_bias": down_b.to(DEV)})
     h = rnd(gen, tokens, width).to(dt)
-    delta = part.forward(h.to(DEV), make_step(dt, [tokens]))
+    start = rnd(gen, tokens, width)
+    stream = ResidualStream(start.clone().to(DEV))
+    assert part.forward(h.to(DEV), make_step(dt, [tokens]), stream) is None
+    stream.flush()
     act = plain.gelu_erf if activation == "gelu_erf" else plain.gelu_tanh
     want = act(h.double() @ up.double().t() + up_b.double()) @ down.double().t() + down_b.double()
-    got = delta.partials.double().sum(0).cpu() + delta.bias.double().cpu()
-    assert rel_err(got, want) < TOL[dtype]
+    assert rel_err(stream.x.cpu().double() - start.double(), want) < TOL[dtype]
     with pytest.raises(ValueError, match="projections are"):
         lookup("feed_forward", "dense")({"width": width, "inner": inner + 8, "activation": activation}, part.tensors)
 
@@ -138,8 +140,10 @@ def test_attention_mixer_alone(dtype, heads, kv_heads, hd, width, window):
         step = make_step(dt, [b - a for a, b in spans], starts=[a for a, _ in spans], cache=cache,
                          slots=[slots[i] for i in live])
         h = torch.cat([xs[i][a:b] for i, (a, b) in zip(live, spans)]).to(DEV)
-        delta = mixer.forward(h, step, Memory(cache, 0, True, step))
-        out = (delta.partials.double().sum(0) + delta.bias.double()).cpu()
+        stream = ResidualStream(torch.zeros(h.shape[0], width, device=DEV))
+        assert mixer.forward(h, step, Memory(cache, 0, True, step), stream) is None
+        stream.flush()
+        out = stream.x.double().cpu()
         at = 0
         for i, (a, b) in zip(live, spans):
             got[i].append(out[at:at + b - a])
@@ -222,7 +226,7 @@ class RunningSumMixer(Mixer):
     def state_spec(self):
         return StateSpec((self.width,), "float32")
 
-    def forward(self, h, step, memory):
+    def forward(self, h, step, memory, stream):
         state = memory.state()
         out = torch.empty(1, h.shape[0], self.width, dtype=torch.float32, device=h.device)
         at = 0

@@ -15,7 +15,9 @@
 // and values of positions that hold no token are replaced by zero before they are multiplied.
 //
 //   attention_prefill  one work-group per (128 queries, head, sequence); each of four waves owns
-//                      32 queries and walks the keys up to its last query's position.
+//                      32 queries (two MFMA column tiles, which share every key and value load)
+//                      and walks the keys up to its last query's position.  (Four column tiles
+//                      per wave were measured and were slower: they leave one wave per SIMD.)
 //   attention_decode   one token per sequence: one work-group per (key/value head, sequence);
 //                      the query heads sharing that head are the MFMA columns; sixteen waves
 //                      (eight for heads above 64) split the keys and meet in LDS.

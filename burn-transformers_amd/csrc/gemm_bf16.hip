@@ -2,10 +2,13 @@
 // accumulation.  Both operands are K-contiguous, which is what an MFMA lane wants: eight
 // consecutive K values in one 16-byte load.
 //
-//   gemm_tile    128 x 128 x 64 tiles for many rows (prefill).  Four waves, each 64 x 64 as
-//                2 x 2 blocks of v_mfma_f32_32x32x16_bf16; operands staged through LDS with an
-//                XOR swizzle of the 16-byte chunks, global loads of the next tile in flight
-//                while the current one is multiplied.
+//   gemm_tile    128 x 128 x 64 tiles for many rows (prefill).  Four waves, each a quarter of the
+//                tile as 2 x 2 blocks of v_mfma_f32_32x32x16_bf16; operands staged through LDS
+//                with an XOR swizzle of the 16-byte chunks, the next tile's global loads in
+//                flight during the multiplication, tiles numbered so that each XCD's L2 sees
+//                neighbours.  (The kernel is a template over the tile and the prefetch depth;
+//                larger tiles and deeper prefetch were measured and lost to this one: they
+//                leave room for one work-group per compute unit only.)
 //   gemm_skinny  up to 64 rows (decode).  The product is bound by streaming W once from HBM:
 //                a work-group owns 16 columns, its eight waves split K, every lane keeps several
 //                16-byte loads of W in flight, v_mfma_f32_16x16x32_bf16 does the arithmetic and
@@ -18,109 +21,165 @@
 #include "host.h"
 #include "epilogue.h"
 
-#define TILE_M 128
-#define TILE_N 128
 #define TILE_K 64
 #define TILE_ROW_BYTES 128
 
 __device__ __forceinline__ int chunks_of(int K) { return (K + 31) / 32; }
 
+// 16-byte chunk `chunk` of row `row` of an LDS tile with 128-byte rows.  The XOR spreads the
+// eight chunks of eight consecutive rows over all banks, so that the 16-byte reads of an MFMA
+// operand (32 consecutive rows, same chunk) do not collide.
 __device__ __forceinline__ int swizzled(int row, int chunk) {
   return row * TILE_ROW_BYTES + ((chunk ^ (row & 7)) << 4);
 }
 
-__global__ void __launch_bounds__(256)
+// Work-groups are handed to the eight XCDs in turn and each XCD has an L2 of its own, so the
+// tiles are renumbered to give every XCD one contiguous range of them; inside a range, tiles
+// that share a block of W's rows come first.
+__device__ __forceinline__ int xcd_contiguous(int bid, int blocks) {
+  int xcd = bid & 7, local = bid >> 3;
+  int q = blocks >> 3, r = blocks & 7;
+  return xcd * q + (xcd < r ? xcd : r) + local;
+}
+
+// BM x BN x 64 tiles, WM x WN waves, each wave (BM / WM) x (BN / WN) as blocks of
+// v_mfma_f32_32x32x16_bf16; LDS holds two stages.  PF register sets hold tiles on their way
+// from memory to LDS: with one, the loads of tile i + 1 fly while tile i is multiplied; with
+// two, tile i + 1 waits in registers and the loads of tile i + 2 fly.
+template <int BM, int BN, int WM, int WN, int PF>
+__global__ void __launch_bounds__(WM * WN * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
-                 int K, Epilogue epi) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2][2][TILE_M * TILE_ROW_BYTES];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int wm = wave & 1, wn = wave >> 1;
+                 int K, Epilogue epi, int tiles_m, int tiles_n) {
+  constexpr int THREADS = WM * WN * 64;
+  constexpr int ROWS = BM + BN;                 // rows of a stage: A's, then W's
+  constexpr int PER_THREAD = ROWS * 8 / THREADS;  // 16-byte chunks a thread moves per tile
+  constexpr int ROW_STEP = THREADS / 8;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  static_assert(ROWS * 8 % THREADS == 0 && BM % ROW_STEP == 0, "tile does not divide among the threads");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][ROWS * 128]
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int wm = wave % WM, wn = wave / WM;
   const int l32 = lane & 31, g = lane >> 5;
-  const int m_base = blockIdx.y * TILE_M, n_base = blockIdx.x * TILE_N;
+  const int tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
+  const int m_base = (tile % tiles_m) * BM, n_base = (tile / tiles_m) * BN;
   const int split = blockIdx.z, splits = gridDim.z;
   const int k_tiles = (K + TILE_K - 1) / TILE_K;
   const int kt_begin = (int)((int64_t)k_tiles * split / splits);
   const int kt_end = (int)((int64_t)k_tiles * (split + 1) / splits);
 
-  // global -> register staging: chunk c of rows r0, r0+32, r0+64, r0+96 of both operands
+  // chunk c of rows r0, r0 + ROW_STEP, ... of the stage: A's rows first, then W's.  Addresses
+  // are rebuilt from the two bases for every load; keeping one pointer per row would not fit
+  // the registers of the larger tiles.
   const int c = tid & 7, r0 = tid >> 3;
-  const bf16_t* a_src[4];
-  const bf16_t* w_src[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int m = m_base + r0 + 32 * i, n = n_base + r0 + 32 * i;
-    m = m < M ? m : M - 1;
-    n = n < N ? n : N - 1;
-    a_src[i] = A + (int64_t)m * lda + c * 8;
-    w_src[i] = W + (int64_t)n * K + c * 8;
-  }
-  uint4 ra[4], rw[4];
-  auto load_tile = [&](int kt) {
+  constexpr int A_CHUNKS = BM / ROW_STEP;
+  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
+  int4v regs[PF][PER_THREAD];
+  auto load_tile = [&](int set, int kt) {
+    // a chunk beyond K (a multiple of 8) reads the row's last chunk and is cleared when stored
     int k = kt * TILE_K + c * 8;
-    bool inside = k < K;
+    int kc = k < K ? k : K - 8;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ra[i] = inside ? *reinterpret_cast<const uint4*>(a_src[i] + kt * TILE_K) : make_uint4(0, 0, 0, 0);
-      rw[i] = inside ? *reinterpret_cast<const uint4*>(w_src[i] + kt * TILE_K) : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < PER_THREAD; ++i) {
+      int row = r0 + ROW_STEP * i;
+      const bf16_t* src;
+      if (i < A_CHUNKS) {
+        int m = m_base + row;
+        src = A + (int64_t)(m < M ? m : M - 1) * lda;
+      } else {
+        int n = n_base + row - BM;
+        src = W + (int64_t)(n < N ? n : N - 1) * K;
+      }
+      regs[set][i] = *reinterpret_cast<const int4v*>(src + kc);
     }
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](int set, int kt, int stage) {
+    int keep = kt * TILE_K + c * 8 < K ? -1 : 0;
+    unsigned char* base = lds + stage * (ROWS * TILE_ROW_BYTES);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int row = r0 + 32 * i;
-      *reinterpret_cast<uint4*>(&lds[buf][0][swizzled(row, c)]) = ra[i];
-      *reinterpret_cast<uint4*>(&lds[buf][1][swizzled(row, c)]) = rw[i];
-    }
+    for (int i = 0; i < PER_THREAD; ++i)
+      *reinterpret_cast<int4v*>(base + swizzled(r0 + ROW_STEP * i, c)) = regs[set][i] & keep;
   };
 
-  floatx16 acc[2][2];
+  floatx16 acc[TN][TM];
 #pragma unroll
-  for (int bn = 0; bn < 2; ++bn)
+  for (int bn = 0; bn < TN; ++bn)
 #pragma unroll
-    for (int bm = 0; bm < 2; ++bm)
+    for (int bm = 0; bm < TM; ++bm)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0.f;
 
-  if (kt_begin < kt_end) {
-    load_tile(kt_begin);
-    store_tile(0);
-  }
-  __syncthreads();
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
-    int buf = (kt - kt_begin) & 1;
-    bool more = kt + 1 < kt_end;
-    if (more) load_tile(kt + 1);
+  auto multiply = [&](int stage) {
+    // all operands of the tile are read before the first multiplication: LDS latency is paid once
+    // per tile, and the reads of later steps return while earlier steps multiply
+    const unsigned char* a_lds = lds + stage * (ROWS * TILE_ROW_BYTES);
+    const unsigned char* w_lds = a_lds + BM * TILE_ROW_BYTES;
+    constexpr int STEPS = TILE_K / 16;
+    bf16x8 wop[STEPS][TN], aop[STEPS][TM];
 #pragma unroll
-    for (int kk = 0; kk < TILE_K / 16; ++kk) {
-      bf16x8 wop[2], aop[2];
+    for (int kk = 0; kk < STEPS; ++kk) {
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        int wrow = wn * 64 + b * 32 + l32, arow = wm * 64 + b * 32 + l32;
-        wop[b] = *reinterpret_cast<const bf16x8*>(&lds[buf][1][swizzled(wrow, 2 * kk + g)]);
-        aop[b] = *reinterpret_cast<const bf16x8*>(&lds[buf][0][swizzled(arow, 2 * kk + g)]);
-      }
+      for (int b = 0; b < TN; ++b)
+        wop[kk][b] = *reinterpret_cast<const bf16x8*>(w_lds + swizzled(wn * (BN / WN) + b * 32 + l32, 2 * kk + g));
 #pragma unroll
-      for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-        for (int bm = 0; bm < 2; ++bm)
-          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wop[bn], aop[bm], acc[bn][bm], 0, 0, 0);
+      for (int b = 0; b < TM; ++b)
+        aop[kk][b] = *reinterpret_cast<const bf16x8*>(a_lds + swizzled(wm * (BM / WM) + b * 32 + l32, 2 * kk + g));
     }
-    if (more) store_tile(buf ^ 1);
+#pragma unroll
+    for (int kk = 0; kk < STEPS; ++kk)
+#pragma unroll
+      for (int bn = 0; bn < TN; ++bn)
+#pragma unroll
+        for (int bm = 0; bm < TM; ++bm)
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wop[kk][bn], aop[kk][bm], acc[bn][bm], 0, 0, 0);
+  };
+
+  const int count = kt_end - kt_begin;
+  if (PF == 1) {
+    // tile i is multiplied from stage i % 2 while the loads of tile i + 1 fly into the registers
+    if (count > 0) {
+      load_tile(0, kt_begin);
+      store_tile(0, kt_begin, 0);
+    }
     __syncthreads();
+    for (int i = 0; i < count; ++i) {
+      if (i + 1 < count) load_tile(0, kt_begin + i + 1);
+      multiply(i & 1);
+      if (i + 1 < count) store_tile(0, kt_begin + i + 1, (i + 1) & 1);
+      __syncthreads();
+    }
+  } else {
+    // tile i is multiplied from stage i % 2 while tile i + 1 sits in register set (i + 1) % 2 and
+    // the loads of tile i + 2 fly into the other set
+    if (count > 0) {
+      load_tile(0, kt_begin);
+      if (count > 1) load_tile(PF - 1, kt_begin + 1);
+      store_tile(0, kt_begin, 0);
+    }
+    __syncthreads();
+    for (int i = 0; i < count; i += 2) {
+      if (i + 2 < count) load_tile(0, kt_begin + i + 2);
+      multiply(0);
+      if (i + 1 < count) store_tile(PF - 1, kt_begin + i + 1, 1);
+      __syncthreads();
+      if (i + 1 >= count) break;
+      if (i + 3 < count) load_tile(PF - 1, kt_begin + i + 3);
+      multiply(1);
+      if (i + 2 < count) store_tile(0, kt_begin + i + 2, 0);
+      __syncthreads();
+    }
   }
 
   // lane holds D[i][j]: i = 8 * (r / 4) + 4 * g + r % 4 (column n), j = lane % 32 (row m)
 #pragma unroll
-  for (int bm = 0; bm < 2; ++bm) {
-    int m = m_base + wm * 64 + bm * 32 + l32;
-    if (m >= M) continue;
+  for (int bm = 0; bm < TM; ++bm) {
+    const int m = m_base + wm * (BM / WM) + bm * 32 + l32;
 #pragma unroll
-    for (int bn = 0; bn < 2; ++bn) {
+    for (int bn = 0; bn < TN; ++bn) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         float v[4] = {acc[bn][bm][4 * q], acc[bn][bm][4 * q + 1], acc[bn][bm][4 * q + 2], acc[bn][bm][4 * q + 3]};
-        int n0 = n_base + wn * 64 + bn * 32 + q * 8 + g * 4;
-        epilogue4<bf16_t>(epi, N, m, n0, v, split);
+        int n0 = n_base + wn * (BN / WN) + bn * 32 + q * 8 + g * 4;
+        if (m < M) epilogue4<bf16_t>(epi, N, m, n0, v, split);
       }
     }
   }
@@ -238,14 +297,27 @@ static int check_operands(const char* who, const void* A, int64_t lda, const voi
   return BT_OK;
 }
 
+template <int BM, int BN, int WM, int WN, int PF>
+static void launch_tile(hipStream_t stream, const bf16_t* A, int64_t lda, const bf16_t* W, int M, int N, int K,
+                        const Epilogue& epi, int splits) {
+  int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  size_t lds = (size_t)2 * (BM + BN) * TILE_ROW_BYTES;
+  auto kernel = gemm_tile_kernel<BM, BN, WM, WN, PF>;
+  if (lds > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, 1, splits), dim3(WM * WN * 64), lds, stream, A, lda, W, M, N,
+                     K, epi, tiles_m, tiles_n);
+}
+
 BT_EXPORT int bt_gemm_tile_bf16(void* stream, const void* A, int64_t lda, const void* W, int M, int N, int K,
                                 const Epilogue* epi, int splits) {
   if (M <= 0) return BT_OK;
   int rc = check_operands("gemm_tile_bf16", A, lda, W, M, N, K, *epi, splits);
   if (rc) return rc;
-  dim3 grid((N + TILE_N - 1) / TILE_N, (M + TILE_M - 1) / TILE_M, splits), block(256);
-  hipLaunchKernelGGL(gemm_tile_kernel, grid, block, 0, (hipStream_t)stream, (const bf16_t*)A, lda,
-                     (const bf16_t*)W, M, N, K, *epi);
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  launch_tile<128, 128, 2, 2, 1>(s, a, lda, w, M, N, K, *epi, splits);
   return bt_check_launch("gemm_tile_bf16");
 }
 

@@ -180,8 +180,10 @@ def gemm(a, w, epilogue, splits=1, impl="auto"):
     if dtype != BFLOAT16:
         raise KernelError(f"gemm: the {impl} kernel takes bfloat16 only")
     lib = _module("gemm_bf16")
-    fn = lib.bt_gemm_tile_bf16 if impl == "tile" else lib.bt_gemm_skinny_bf16
-    _check(lib, fn(_c_ptr(_stream()), *args, _c_int(splits)))
+    if impl == "tile":
+        _check(lib, lib.bt_gemm_tile_bf16(_c_ptr(_stream()), *args, _c_int(splits)))
+    else:
+        _check(lib, lib.bt_gemm_skinny_bf16(_c_ptr(_stream()), *args, _c_int(splits)))
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,

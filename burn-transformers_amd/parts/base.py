@@ -45,9 +45,9 @@ class ResidualStream:
         self.pending = delta
 
     def add_product(self, step, a, weight, bias=None):
-        """x += a . weight^T + bias.  With bfloat16 and up to 64 rows (decode) the product splits its K
-        range into partial sums that stay pending: a weight-streaming product with few output columns
-        needs the extra work-groups to pull its matrix through HBM.  Otherwise the product's epilogue
+        """x += a . weight^T + bias.  With bfloat16 a product with few output columns splits its K range
+        into partial sums that stay pending: in decode the extra work-groups are needed to pull the
+        matrix through HBM, in prefill to occupy all compute units.  Otherwise the product's epilogue
         adds into the stream in place."""
         rows, width = a.shape[0], weight.shape[0]
         splits = split_count(rows, width, a.shape[1]) if step.dtype_is_bf16 else 1
@@ -137,10 +137,14 @@ class Block:
 
 
 def split_count(rows, columns, k):
-    """How many ways a residual-writing product splits its K range in decode: few output columns
-    give too few work-groups to pull a weight matrix through HBM at full rate."""
+    """How many ways a residual-writing product splits its K range."""
     if rows > 64:
-        return 1
+        # prefill: 128 x 128 tiles; few output columns leave compute units idle unless K is split
+        tiles = ((rows + 127) // 128) * ((columns + 127) // 128)
+        splits = 1
+        while tiles * splits < 512 and splits < 4 and k // (splits * 2) >= 512:
+            splits *= 2
+        return splits
     tiles = (columns + 15) // 16
     splits = 1
     # at least as many work-groups as compute units (256), and still a few chunks of 32 for

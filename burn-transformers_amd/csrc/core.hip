@@ -94,42 +94,48 @@ __global__ void add_norm_kernel(float* __restrict__ x, const float* __restrict__
   }
 }
 
-// The same for rows whose width is a multiple of four and at most 1024 * VPT (VPT up to 4): the row lives
-// in registers, every load of a thread (stream, each partial sum, bias) is independent of the
-// others and in flight at once.  A decode step has few rows, so one row's latency is what counts.
-#define ADD_NORM_MAX_SPLITS 8
-template <typename T, int VPT>
+// The same for rows whose width is a multiple of four and at most 1024 * VPT (VPT up to 4), with
+// exactly NS partial sums: the row lives in registers and the code is straight-line, so every
+// load of a thread (stream, each partial sum, bias, scale, shift) is a 16-byte load that is in
+// flight together with all the others.  A decode step has few rows: one row's latency counts.
+// Zeros to read where a bias or a shift is absent: selecting the pointer keeps the loads
+// unconditional (a test of the pointer around each load would split them into pieces).
+__device__ float bt_zero_row[4096];
+
+template <typename T, int VPT, int NS>
 __global__ void __launch_bounds__(256)
-add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int n_delta,
-                    int64_t delta_stride, const float* __restrict__ bias, const float* __restrict__ gamma,
+add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int64_t delta_stride,
+                    const float* __restrict__ bias, const float* __restrict__ gamma,
                     const float* __restrict__ beta, float eps, int kind, T* __restrict__ out,
                     const int* __restrict__ rows, int width, int write_back) {
   __shared__ float scratch[32];
   const int r = blockIdx.x;
   const int t = rows ? rows[r] : r;
   const int quads = width >> 2;
-  float4* xr = reinterpret_cast<float4*>(x + (int64_t)t * width);
-  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-  float4 v[VPT], part[VPT][ADD_NORM_MAX_SPLITS], b[VPT], g[VPT], be[VPT];
-  // every load of the kernel is issued here, before anything waits: one trip to memory
+  float4* xr = reinterpret_cast<float4*>(x) + (int64_t)t * quads;
+  const float4* dr = reinterpret_cast<const float4*>(delta) + (int64_t)t * quads;
+  const int64_t dstride = delta_stride >> 2;
+  const float4* z4 = reinterpret_cast<const float4*>(bt_zero_row);
+  const float4* b4 = bias ? reinterpret_cast<const float4*>(bias) : z4;
+  const float4* g4 = gamma ? reinterpret_cast<const float4*>(gamma) : z4;
+  const float4* be4 = beta ? reinterpret_cast<const float4*>(beta) : z4;
+  float4 v[VPT], part[VPT][NS > 0 ? NS : 1], b[VPT], g[VPT], be[VPT];
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     int c = threadIdx.x + i * 256;
-    int cc = c < quads ? c : 0;
+    int cc = c < quads ? c : 0;     // lanes beyond the row read column 0; the result is never used
     v[i] = xr[cc];
-    b[i] = bias ? reinterpret_cast<const float4*>(bias)[cc] : zero;
-    g[i] = (out != nullptr) ? reinterpret_cast<const float4*>(gamma)[cc] : zero;
-    be[i] = (out != nullptr && beta) ? reinterpret_cast<const float4*>(beta)[cc] : zero;
 #pragma unroll
-    for (int s = 0; s < ADD_NORM_MAX_SPLITS; ++s)
-      part[i][s] = (s < n_delta) ? reinterpret_cast<const float4*>(delta + s * delta_stride + (int64_t)t * width)[cc]
-                                 : zero;
-  }   // lanes beyond the row read column 0; whatever they hold is never used below
+    for (int s = 0; s < NS; ++s) part[i][s] = dr[s * dstride + cc];
+    b[i] = b4[cc];
+    g[i] = g4[cc];
+    be[i] = be4[cc];
+  }
   float partial = 0.f;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
 #pragma unroll
-    for (int s = 0; s < ADD_NORM_MAX_SPLITS; ++s) {   // same order of additions as the plain kernel
+    for (int s = 0; s < NS; ++s) {   // same order of additions as the plain kernel
       v[i].x += part[i][s].x; v[i].y += part[i][s].y; v[i].z += part[i][s].z; v[i].w += part[i][s].w;
     }
     v[i].x += b[i].x; v[i].y += b[i].y; v[i].z += b[i].z; v[i].w += b[i].w;
@@ -140,6 +146,7 @@ add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int 
                              : (v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w);
     }
   }
+  if (out == nullptr) return;
   float total = block_sum(partial, scratch);
   float mean = 0.f, rstd;
   if (kind == 0) {
@@ -157,7 +164,6 @@ add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int 
   } else {
     rstd = 1.0f / sqrtf(total / (float)width + eps);
   }
-  if (out == nullptr) return;
   T* orow = out + (int64_t)r * width;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
@@ -169,22 +175,42 @@ add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int 
   }
 }
 
+template <typename T, int VPT>
+static bool launch_add_norm_vec(hipStream_t stream, dim3 grid, float* x, const float* delta, int n_delta,
+                                int64_t delta_stride, const float* bias, const float* gamma, const float* beta,
+                                float eps, int kind, T* out, const int* rows, int width, int write_back) {
+#define BT_ADD_NORM_VEC(NS)                                                                                  \
+  hipLaunchKernelGGL((add_norm_vec_kernel<T, VPT, NS>), grid, dim3(256), 0, stream, x, delta, delta_stride,  \
+                     bias, gamma, beta, eps, kind, out, rows, width, write_back)
+  switch (n_delta) {
+    case 0: BT_ADD_NORM_VEC(0); return true;
+    case 1: BT_ADD_NORM_VEC(1); return true;
+    case 2: BT_ADD_NORM_VEC(2); return true;
+    case 4: BT_ADD_NORM_VEC(4); return true;
+    case 8: BT_ADD_NORM_VEC(8); return true;
+    default: return false;
+  }
+#undef BT_ADD_NORM_VEC
+}
+
 template <typename T>
 static void launch_add_norm(hipStream_t stream, float* x, const float* delta, int n_delta, int64_t delta_stride,
                             const float* bias, const float* gamma, const float* beta, float eps, int kind,
                             T* out, const int* rows, int n_rows, int width, int write_back) {
-  dim3 grid(n_rows), block(256);
-  bool vec = width % 4 == 0 && width <= 4096 && n_delta <= ADD_NORM_MAX_SPLITS && delta_stride % 4 == 0;
-#define BT_ADD_NORM_VEC(VPT)                                                                             \
-  hipLaunchKernelGGL((add_norm_vec_kernel<T, VPT>), grid, block, 0, stream, x, delta, n_delta, delta_stride, \
-                     bias, gamma, beta, eps, kind, out, rows, width, write_back)
-  if (vec && width <= 1024) BT_ADD_NORM_VEC(1);
-  else if (vec && width <= 2048) BT_ADD_NORM_VEC(2);
-  else if (vec) BT_ADD_NORM_VEC(4);
-  else
-    hipLaunchKernelGGL(add_norm_kernel<T>, grid, block, (size_t)width * sizeof(float), stream, x, delta,
+  dim3 grid(n_rows);
+  auto aligned = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  bool vec = width % 4 == 0 && width <= 4096 && delta_stride % 4 == 0 && aligned(x) && aligned(delta) &&
+             aligned(bias) && aligned(gamma) && aligned(beta) && aligned(out);
+  bool done = false;
+  if (vec && width <= 1024)
+    done = launch_add_norm_vec<T, 1>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+  else if (vec && width <= 2048)
+    done = launch_add_norm_vec<T, 2>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+  else if (vec)
+    done = launch_add_norm_vec<T, 4>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+  if (!done)
+    hipLaunchKernelGGL(add_norm_kernel<T>, grid, dim3(256), (size_t)width * sizeof(float), stream, x, delta,
                        n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
-#undef BT_ADD_NORM_VEC
 }
 
 BT_EXPORT int bt_add_norm(void* stream, int out_dtype, float* x, const float* delta, int n_delta,

@@ -26,11 +26,14 @@
 
 __device__ __forceinline__ int chunks_of(int K) { return (K + 31) / 32; }
 
-// 16-byte chunk `chunk` of row `row` of an LDS tile with 128-byte rows.  The XOR spreads the
-// eight chunks of eight consecutive rows over all banks, so that the 16-byte reads of an MFMA
-// operand (32 consecutive rows, same chunk) do not collide.
+// 16-byte chunk `chunk` of row `row` of an LDS tile with 128-byte rows.  LDS has 64 banks of four
+// bytes and serves 16 lanes of a 16-byte access at a time, so two rows span the banks once and
+// the 16 consecutive rows that read the same chunk for an MFMA operand must land in 16 different
+// 16-byte slots: the chunk is XORed with bits 1..3 of the row (rows 2j and 2j + 1 share a value
+// and differ in the half of the banks they occupy).  Measured with SQ_LDS_BANK_CONFLICT: a third
+// of the LDS cycles were conflicts with the XOR taken from bits 0..2.
 __device__ __forceinline__ int swizzled(int row, int chunk) {
-  return row * TILE_ROW_BYTES + ((chunk ^ (row & 7)) << 4);
+  return row * TILE_ROW_BYTES + ((chunk ^ ((row >> 1) & 7)) << 4);
 }
 
 // Work-groups are handed to the eight XCDs in turn and each XCD has an L2 of its own, so the
@@ -185,6 +188,248 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
   }
 }
 
+// The same 128 x 128 x 64 tiling for K a multiple of 64 and operands below 4 GiB, written so that
+// the loop over K holds almost nothing but loads, LDS traffic and MFMAs.  Counters
+// (SQ_INSTS_VALU against SQ_INSTS_VALU_MFMA_MOPS) showed five ordinary vector instructions per
+// MFMA in the template above, nearly all of them address arithmetic.  Here every address is a
+// uniform base that a scalar add advances, plus a per-lane offset computed once: global loads
+// take a 32-bit lane offset, LDS accesses one lane offset plus an immediate (rows 32 apart share
+// their swizzle and lie 4096 bytes apart; the two stages are 32 KiB apart).
+#define FAST_STAGE_BYTES (256 * TILE_ROW_BYTES)
+#define FAST_W_BYTES (128 * TILE_ROW_BYTES)
+
+__global__ void __launch_bounds__(256)
+gemm_tile_fast_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
+                      int K, Epilogue epi, int tiles_m, int tiles_n) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * FAST_STAGE_BYTES];
+  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
+  const int m_base = (tile % tiles_m) * 128, n_base = (tile / tiles_m) * 128;
+  const int split = blockIdx.z, splits = gridDim.z;
+  const int k_tiles = K / TILE_K;
+  const int kt_begin = (int)((int64_t)k_tiles * split / splits);
+  const int count = (int)((int64_t)k_tiles * (split + 1) / splits) - kt_begin;
+
+  const int c = tid & 7, r0 = tid >> 3;
+  unsigned a_off[4], w_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int m = m_base + r0 + 32 * i, n = n_base + r0 + 32 * i;
+    m = m < M ? m : M - 1;
+    n = n < N ? n : N - 1;
+    a_off[i] = (unsigned)(((int64_t)m * lda + c * 8) * 2);
+    w_off[i] = (unsigned)(((int64_t)n * K + c * 8) * 2);
+  }
+  const unsigned char* a_k = reinterpret_cast<const unsigned char*>(A) + (int64_t)kt_begin * (TILE_K * 2);
+  const unsigned char* w_k = reinterpret_cast<const unsigned char*>(W) + (int64_t)kt_begin * (TILE_K * 2);
+  const int st_off = swizzled(r0, c);
+  int w_rd[4], a_rd[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    w_rd[kk] = FAST_W_BYTES + swizzled(wn * 64 + l32, 2 * kk + g);
+    a_rd[kk] = swizzled(wm * 64 + l32, 2 * kk + g);
+  }
+
+  int4v ra[4], rw[4];
+  auto load_tile = [&]() {     // the tile a_k, w_k point at; then advance them
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ra[i] = *reinterpret_cast<const int4v*>(a_k + a_off[i]);
+      rw[i] = *reinterpret_cast<const int4v*>(w_k + w_off[i]);
+    }
+    a_k += TILE_K * 2;
+    w_k += TILE_K * 2;
+  };
+  auto store_tile = [&](int stage_bytes) {
+    unsigned char* base = lds + stage_bytes + st_off;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<int4v*>(base + i * 4096) = ra[i];
+      *reinterpret_cast<int4v*>(base + FAST_W_BYTES + i * 4096) = rw[i];
+    }
+  };
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+    for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0.f;
+
+  if (count > 0) {
+    load_tile();
+    store_tile(0);
+  }
+  __syncthreads();
+  // one loop body, no exit in its middle: the accumulators then stay where the MFMAs want them
+  // (with the loop unrolled by two and left from its middle, the compiler copied all of them
+  // between register files in every iteration)
+  int stage_bytes = 0;
+  for (int i = 0; i < count; ++i) {
+    const bool more = i + 1 < count;
+    if (more) load_tile();
+    const unsigned char* base = lds + stage_bytes;
+    bf16x8 wop[4][2], aop[4][2];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        wop[kk][b] = *reinterpret_cast<const bf16x8*>(base + w_rd[kk] + b * 4096);
+        aop[kk][b] = *reinterpret_cast<const bf16x8*>(base + a_rd[kk] + b * 4096);
+      }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int bm = 0; bm < 2; ++bm)
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wop[kk][bn], aop[kk][bm], acc[bn][bm], 0, 0, 0);
+    stage_bytes ^= FAST_STAGE_BYTES;
+    if (more) store_tile(stage_bytes);
+    __syncthreads();
+  }
+
+  // lane holds D[i][j]: i = 8 * (r / 4) + 4 * g + r % 4 (column n), j = lane % 32 (row m)
+#pragma unroll
+  for (int bm = 0; bm < 2; ++bm) {
+    const int m = m_base + wm * 64 + bm * 32 + l32;
+#pragma unroll
+    for (int bn = 0; bn < 2; ++bn) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float v[4] = {acc[bn][bm][4 * q], acc[bn][bm][4 * q + 1], acc[bn][bm][4 * q + 2], acc[bn][bm][4 * q + 3]};
+        int n0 = n_base + wn * 64 + bn * 32 + q * 8 + g * 4;
+        if (m < M) epilogue4<bf16_t>(epi, N, m, n0, v, split);
+      }
+    }
+  }
+}
+
+// The third form of the same tiling moves the operands from memory straight into LDS
+// (global_load_lds_dwordx4: every lane names 16 bytes in memory, the wave's 64 pieces land in one
+// contiguous KiB of LDS), which frees the staging registers and, more to the point, lets
+// DMA_STAGES - 1 tiles be in flight while one is multiplied: the products above are bound by
+// memory latency (one tile in flight per work-group, two work-groups per compute unit), not by
+// MFMA or LDS throughput.  The compiler's own bookkeeping would wait for ALL such loads before any
+// LDS read, so the waits are written by hand (s_waitcnt vmcnt(n) with n = loads of the tiles that
+// may still be in flight) and the work-group meets at a bare s_barrier:
+//     wait for my loads of tile i | barrier | start the loads of tile i + STAGES - 1 into the
+//     stage tile i - 1 was read from | read tile i from LDS | multiply
+// The swizzle is applied on the memory side: lane l of the load that fills rows 8 s .. 8 s + 7
+// writes physical chunk l % 8 of row 8 s + l / 8, so it fetches the logical chunk that belongs
+// there.  K must be a multiple of 64, operands below 4 GiB.
+#define DMA_STAGES 4
+#define DMA_LOADS 8   // global_load_lds instructions per wave and tile
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__global__ void __launch_bounds__(256)
+gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
+                     int K, Epilogue epi, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [DMA_STAGES][256 rows][128 bytes]
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
+  const int m_base = (tile % tiles_m) * 128, n_base = (tile / tiles_m) * 128;
+  const int split = blockIdx.z, splits = gridDim.z;
+  const int k_tiles = K / TILE_K;
+  const int kt_begin = (int)((int64_t)k_tiles * split / splits);
+  const int count = (int)((int64_t)k_tiles * (split + 1) / splits) - kt_begin;
+
+  // waves 0 and 1 fetch A's 128 rows, waves 2 and 3 W's: load j of a wave fills stage rows
+  // 64 * wave + 8 j .. + 7 (rows 128 .. 255 of a stage are W's)
+  const bool fetch_w = wave >= 2;
+  const unsigned char* src = reinterpret_cast<const unsigned char*>(fetch_w ? W : A) +
+                             (int64_t)kt_begin * (TILE_K * 2);
+  unsigned off[DMA_LOADS];
+#pragma unroll
+  for (int j = 0; j < DMA_LOADS; ++j) {
+    int stage_row = 64 * wave + 8 * j + (lane >> 3);
+    int chunk = (lane & 7) ^ ((stage_row >> 1) & 7);
+    int row = (stage_row & 127) + (fetch_w ? n_base : m_base);
+    int limit = fetch_w ? N : M;
+    row = row < limit ? row : limit - 1;
+    off[j] = (unsigned)(((int64_t)row * (fetch_w ? (int64_t)K : lda) + chunk * 8) * 2);
+  }
+  auto issue = [&](int stage) {   // the tile `src` points at, into `stage`; then advance
+#pragma unroll
+    for (int j = 0; j < DMA_LOADS; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(src + off[j]),
+          (__attribute__((address_space(3))) void*)(lds + stage * FAST_STAGE_BYTES + (64 * wave + 8 * j) * TILE_ROW_BYTES),
+          16, 0, 0);
+    src += TILE_K * 2;
+  };
+  int w_rd[4], a_rd[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    w_rd[kk] = FAST_W_BYTES + swizzled(wn * 64 + l32, 2 * kk + g);
+    a_rd[kk] = swizzled(wm * 64 + l32, 2 * kk + g);
+  }
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+    for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0.f;
+
+#pragma unroll
+  for (int t = 0; t < DMA_STAGES - 1; ++t)
+    if (t < count) issue(t);
+  int stage = 0, next_stage = DMA_STAGES - 1;
+  for (int i = 0; i < count; ++i) {
+    // tiles i + 1 .. i + STAGES - 2 (those that exist) may still be in flight
+    int newer = count - 1 - i;
+    if (newer >= DMA_STAGES - 2) wait_vmcnt<DMA_LOADS * (DMA_STAGES - 2)>();
+    else if (newer == 1) wait_vmcnt<DMA_LOADS>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (i + DMA_STAGES - 1 < count) issue(next_stage);
+    const unsigned char* base = lds + stage * FAST_STAGE_BYTES;
+    bf16x8 wop[4][2], aop[4][2];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        wop[kk][b] = *reinterpret_cast<const bf16x8*>(base + w_rd[kk] + b * 4096);
+        aop[kk][b] = *reinterpret_cast<const bf16x8*>(base + a_rd[kk] + b * 4096);
+      }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int bm = 0; bm < 2; ++bm)
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wop[kk][bn], aop[kk][bm], acc[bn][bm], 0, 0, 0);
+    stage = stage + 1 == DMA_STAGES ? 0 : stage + 1;
+    next_stage = next_stage + 1 == DMA_STAGES ? 0 : next_stage + 1;
+  }
+
+  // lane holds D[i][j]: i = 8 * (r / 4) + 4 * g + r % 4 (column n), j = lane % 32 (row m)
+#pragma unroll
+  for (int bm = 0; bm < 2; ++bm) {
+    const int m = m_base + wm * 64 + bm * 32 + l32;
+#pragma unroll
+    for (int bn = 0; bn < 2; ++bn) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float v[4] = {acc[bn][bm][4 * q], acc[bn][bm][4 * q + 1], acc[bn][bm][4 * q + 2], acc[bn][bm][4 * q + 3]};
+        int n0 = n_base + wn * 64 + bn * 32 + q * 8 + g * 4;
+        if (m < M) epilogue4<bf16_t>(epi, N, m, n0, v, split);
+      }
+    }
+  }
+}
+
 // Memory latency on this GPU is about a microsecond and one compute unit alone pulls only a few
 // per cent of the HBM bandwidth, while a decode step is hundreds of short kernels.  So the
 // skinny kernel (a) wants at least as many work-groups as there are compute units, which is
@@ -309,15 +554,41 @@ static void launch_tile(hipStream_t stream, const bf16_t* A, int64_t lda, const 
                      K, epi, tiles_m, tiles_n);
 }
 
+// variant: 0 = the fastest form the operands allow; 1 = template, 2 = lean, 3 = direct to LDS
+// (asked for by tests and measurements; a form that cannot take the operands is refused)
 BT_EXPORT int bt_gemm_tile_bf16(void* stream, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                                const Epilogue* epi, int splits) {
+                                const Epilogue* epi, int splits, int variant) {
   if (M <= 0) return BT_OK;
   int rc = check_operands("gemm_tile_bf16", A, lda, W, M, N, K, *epi, splits);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  launch_tile<128, 128, 2, 2, 1>(s, a, lda, w, M, N, K, *epi, splits);
+  const int64_t four_gib = (int64_t)1 << 32;
+  const bool lean_ok = K % TILE_K == 0 && (int64_t)M * lda * 2 < four_gib && (int64_t)N * K * 2 < four_gib;
+  // Direct to LDS keeps three tiles in flight but leaves room for one work-group per compute
+  // unit; it wins when there is at most one tile per compute unit anyway, the lean form (two
+  // work-groups per unit) when there are more.
+  if (variant == 0) variant = !lean_ok ? 1 : ((int64_t)((M + 127) / 128) * ((N + 127) / 128) * splits <= 256 ? 3 : 2);
+  if (variant != 1 && !lean_ok)
+    BT_REFUSE("gemm_tile_bf16: this form needs K %d to be a multiple of 64 and operands below 4 GiB", K);
+  int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
+  dim3 grid(tiles_m * tiles_n, 1, splits);
+  if (variant == 3) {
+    size_t lds = (size_t)DMA_STAGES * FAST_STAGE_BYTES;
+    static bool raised = false;
+    if (!raised) {
+      hipError_t err = hipFuncSetAttribute((const void*)gemm_tile_dma_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (err != hipSuccess) BT_REFUSE("gemm_tile_bf16: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));
+      raised = true;
+    }
+    hipLaunchKernelGGL(gemm_tile_dma_kernel, grid, dim3(256), lds, s, a, lda, w, M, N, K, *epi, tiles_m, tiles_n);
+  } else if (variant == 2) {
+    hipLaunchKernelGGL(gemm_tile_fast_kernel, grid, dim3(256), 0, s, a, lda, w, M, N, K, *epi, tiles_m, tiles_n);
+  } else {
+    launch_tile<128, 128, 2, 2, 1>(s, a, lda, w, M, N, K, *epi, splits);
+  }
   return bt_check_launch("gemm_tile_bf16");
 }
 

@@ -156,11 +156,12 @@ def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None,
         _c_int(1 if write_back else 0)))
 
 
-def gemm(a, w, epilogue, splits=1, impl="auto"):
+def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
     """C = a . w^T handed to ``epilogue``.  a: [M, K] (rows may be strided), w: [N, K] contiguous.
 
     impl: "auto" (float32 -> plain; bfloat16 -> skinny up to 64 rows, else tile), or one of
-    "plain", "tile", "skinny" to force a kernel.
+    "plain", "tile", "skinny" to force a kernel.  variant picks one of the tile kernel's forms
+    (0: the fastest the operands allow, 1: any K, 2: lean, 3: direct to LDS).
     """
     m, k = a.shape
     n = w.shape[0]
@@ -181,7 +182,7 @@ def gemm(a, w, epilogue, splits=1, impl="auto"):
         raise KernelError(f"gemm: the {impl} kernel takes bfloat16 only")
     lib = _module("gemm_bf16")
     if impl == "tile":
-        _check(lib, lib.bt_gemm_tile_bf16(_c_ptr(_stream()), *args, _c_int(splits)))
+        _check(lib, lib.bt_gemm_tile_bf16(_c_ptr(_stream()), *args, _c_int(splits), _c_int(variant)))
     else:
         _check(lib, lib.bt_gemm_skinny_bf16(_c_ptr(_stream()), *args, _c_int(splits)))
 

@@ -45,10 +45,10 @@ class ResidualStream:
         self.pending = delta
 
     def add_product(self, step, a, weight, bias=None):
-        """x += a . weight^T + bias.  With bfloat16 a product with few output columns splits its K range
-        into partial sums that stay pending: in decode the extra work-groups are needed to pull the
-        matrix through HBM, in prefill to occupy all compute units.  Otherwise the product's epilogue
-        adds into the stream in place."""
+        """x += a . weight^T + bias.  In a bfloat16 decode step (up to 64 rows) a product with few
+        output columns splits its K range into partial sums that stay pending: the extra work-groups
+        are needed to pull the matrix through HBM.  Otherwise the product's epilogue adds into the
+        stream in place."""
         rows, width = a.shape[0], weight.shape[0]
         splits = split_count(rows, width, a.shape[1]) if step.dtype_is_bf16 else 1
         if splits > 1:
@@ -139,12 +139,7 @@ class Block:
 def split_count(rows, columns, k):
     """How many ways a residual-writing product splits its K range."""
     if rows > 64:
-        # prefill: 128 x 128 tiles; few output columns leave compute units idle unless K is split
-        tiles = ((rows + 127) // 128) * ((columns + 127) // 128)
-        splits = 1
-        while tiles * splits < 512 and splits < 4 and k // (splits * 2) >= 512:
-            splits *= 2
-        return splits
+        return 1
     tiles = (columns + 15) // 16
     splits = 1
     # at least as many work-groups as compute units (256), and still a few chunks of 32 for

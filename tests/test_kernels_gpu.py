@@ -55,6 +55,24 @@ def test_gemm_epilogues(impl, dtype, m, n, k):
     assert rel_err(out32, want) < (2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k))
 
 
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (300, 517, 1600), (130, 96, 192), (1000, 1600, 6400)])
+def test_tile_gemm_forms_agree(variant, m, n, k):
+    """The three forms of the tile kernel (any K; lean; direct to LDS) against float64."""
+    a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=variant, lda=k + 64)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K.gemm(a, w, K.epilogue_act(out, "gelu_erf", bias), impl="tile", variant=variant)
+    assert rel_err(out, gelu_erf(want + bias.cpu().double())) < 6e-3
+    parts = torch.full((3, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    K.gemm(a, w, K.epilogue_f32(parts), impl="tile", variant=variant, splits=3)
+    assert rel_err(parts.sum(0), want) < 2e-5 * math.sqrt(k)
+    if variant > 1:
+        a2, w2, _, _ = operands(70, 40, 96, torch.bfloat16)
+        with pytest.raises(K.KernelError, match="multiple of 64"):
+            K.gemm(a2, w2, K.epilogue_store(torch.empty(70, 40, dtype=torch.bfloat16, device=DEV)), impl="tile",
+                   variant=variant)
+
+
 @pytest.mark.parametrize("impl,m,n,k,splits", [("skinny", 5, 96, 1600, 4), ("skinny", 64, 50, 6400, 8),
                                                ("skinny", 20, 1600, 320, 2), ("tile", 150, 200, 1600, 3)])
 def test_gemm_split_k_partials(impl, m, n, k, splits):

@@ -233,21 +233,34 @@ attention_decode_kernel(AttnArgs a) {
   float* sm_m = sm;                                   // [DECODE_WAVES][group]
   float* sm_l = sm + DECODE_WAVES * group;            // [DECODE_WAVES][group]
   float* sm_o = sm + 2 * DECODE_WAVES * group;        // [DECODE_WAVES][group][HD]
-  const int tok = a.seq_off[seq], pos = a.seq_start[seq];
+  // One token per sequence, in the order of the sequences: token `seq` belongs to sequence `seq`.
+  // The query, the position and (without a window) the blocks of this wave's first two tiles do
+  // not depend on each other, so their loads fly together; the keys and values then need one
+  // more trip to memory, not two.
+  const int tok = seq;
   const bf16_t* Q = static_cast<const bf16_t*>(a.q);
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const bool has_query = i16 < group;
   const int head = kv_head * group + (has_query ? i16 : 0);
-
-  int qpos[1] = {has_query ? pos : -1};
+  const int stride = 32 * DECODE_WAVES;
+  const int* block_row = a.kv.blocks + (int64_t)seq * a.kv.max_blocks;
+  const int last_entry = a.kv.max_blocks - 1;
+  int early_block0 = 0, early_block1 = 0;
+  if (a.window == 0) {
+    int entry0 = (32 * wave) / BT_KV_BLOCK, entry1 = (32 * wave + stride) / BT_KV_BLOCK;
+    early_block0 = block_row[entry0 < last_entry ? entry0 : last_entry];
+    early_block1 = block_row[entry1 < last_entry ? entry1 : last_entry];
+  }
+  const int pos = a.seq_start[seq];
   bf16x8 q[1][NKS];
-  floatx4 o[1][ND];
-  float m[1] = {-INFINITY}, l[1] = {0.f};
 #pragma unroll
   for (int ks = 0; ks < NKS; ++ks) {
     int channel = ks * 32 + g * 8;
     q[0][ks] = (has_query && channel < HD) ? load_bf16x8(Q + (int64_t)tok * a.ldq + head * HD + channel) : zero8;
   }
+  int qpos[1] = {has_query ? pos : -1};
+  floatx4 o[1][ND];
+  float m[1] = {-INFINITY}, l[1] = {0.f};
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt) o[0][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
@@ -255,16 +268,22 @@ attention_decode_kernel(AttnArgs a) {
   if (a.window > 0 && pos - a.window + 1 > 0) lo = (pos - a.window + 1) & ~31;
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
-  const int first = lo + 32 * wave, stride = 32 * DECODE_WAVES;
+  const int first = lo + 32 * wave;
+  // plane of the tile at kb: from the blocks fetched early where they apply, else from the table
+  auto plane_of = [&](int kb, int j) {
+    int block = (a.window == 0 && j < 2) ? (j == 0 ? early_block0 : early_block1) : block_row[kb / BT_KV_BLOCK];
+    return ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
+  };
   TileOperands current, next;
   if (first <= pos) {
-    int64_t plane = tile_plane(a, seq, kv_head, first);
+    int64_t plane = plane_of(first, 0);
     load_tile(next, keys + plane, values + plane, first);
   }
-  for (int kb = first; kb <= pos; kb += stride) {
+  int j = 0;
+  for (int kb = first; kb <= pos; kb += stride, ++j) {
     current = next;
     if (kb + stride <= pos) {
-      int64_t plane = tile_plane(a, seq, kv_head, kb + stride);
+      int64_t plane = plane_of(kb + stride, j + 1);
       load_tile(next, keys + plane, values + plane, kb + stride);
     }
     attend_tile<1>(current, kb, pos + 1, qpos, a.window, a.scale, q, o, m, l);

@@ -73,6 +73,21 @@ def test_tile_gemm_forms_agree(variant, m, n, k):
                    variant=variant)
 
 
+@pytest.mark.parametrize("m,n,k,splits", [(1, 100, 136, 1), (8, 4800, 1600, 2), (16, 1600, 1600, 4),
+                                          (7, 333, 6400, 8), (3, 50, 1760, 1), (16, 517, 1608, 3),
+                                          (2, 16, 8, 1), (9, 40, 3400, 1)])
+def test_skinny_gemm_at_decode_sizes(m, n, k, splits):
+    """Up to 16 rows, K with a short last chunk, slices of K that do not divide evenly."""
+    a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=k, lda=k + 24)
+    parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl="skinny")
+    assert rel_err(parts.sum(0), want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
+    if splits == 1:
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        K.gemm(a, w, K.epilogue_act(out, "gelu_tanh", bias), impl="skinny")
+        assert rel_err(out, gelu_tanh(want + bias.cpu().double())) < 6e-3
+
+
 @pytest.mark.parametrize("impl,m,n,k,splits", [("skinny", 5, 96, 1600, 4), ("skinny", 64, 50, 6400, 8),
                                                ("skinny", 20, 1600, 320, 2), ("tile", 150, 200, 1600, 3)])
 def test_gemm_split_k_partials(impl, m, n, k, splits):

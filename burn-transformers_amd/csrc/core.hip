@@ -186,7 +186,11 @@ static bool launch_add_norm_vec(hipStream_t stream, dim3 grid, float* x, const f
     case 0: BT_ADD_NORM_VEC(0); return true;
     case 1: BT_ADD_NORM_VEC(1); return true;
     case 2: BT_ADD_NORM_VEC(2); return true;
+    case 3: BT_ADD_NORM_VEC(3); return true;
     case 4: BT_ADD_NORM_VEC(4); return true;
+    case 5: BT_ADD_NORM_VEC(5); return true;
+    case 6: BT_ADD_NORM_VEC(6); return true;
+    case 7: BT_ADD_NORM_VEC(7); return true;
     case 8: BT_ADD_NORM_VEC(8); return true;
     default: return false;
   }

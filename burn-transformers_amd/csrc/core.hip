@@ -175,6 +175,84 @@ add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int6
   }
 }
 
+// The same for steps with many rows (a prefill): one WAVE per row, four rows per work-group.  The
+// row lives in the wave's registers (QPL quads of four floats per lane, so width <= 256 * QPL),
+// statistics are wave reductions with no barrier, and a compute unit has many rows in flight;
+// with one work-group per row the two block-wide reductions leave the memory system idle.
+template <typename T, int QPL>
+__global__ void __launch_bounds__(256)
+add_norm_rows_kernel(float* __restrict__ x, const float* __restrict__ delta, int n_delta, int64_t delta_stride,
+                     const float* __restrict__ bias, const float* __restrict__ gamma,
+                     const float* __restrict__ beta, float eps, int kind, T* __restrict__ out,
+                     const int* __restrict__ rows, int n_rows, int width, int write_back) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + wave;
+  if (r >= n_rows) return;                     // a whole wave leaves; there is no barrier below
+  const int t = rows ? rows[r] : r;
+  const int quads = width >> 2;
+  float4* xr = reinterpret_cast<float4*>(x) + (int64_t)t * quads;
+  const float4* dr = reinterpret_cast<const float4*>(delta) + (int64_t)t * quads;
+  const int64_t dstride = delta_stride >> 2;
+  const float4* z4 = reinterpret_cast<const float4*>(bt_zero_row);
+  const float4* b4 = bias ? reinterpret_cast<const float4*>(bias) : z4;
+  const float4* g4 = gamma ? reinterpret_cast<const float4*>(gamma) : z4;
+  const float4* be4 = beta ? reinterpret_cast<const float4*>(beta) : z4;
+  float4 v[QPL];
+#pragma unroll
+  for (int i = 0; i < QPL; ++i) {
+    int c = lane + i * 64;
+    v[i] = xr[c < quads ? c : 0];
+  }
+  for (int s = 0; s < n_delta; ++s) {          // same order of additions as the plain kernel
+#pragma unroll
+    for (int i = 0; i < QPL; ++i) {
+      int c = lane + i * 64;
+      float4 d = dr[s * dstride + (c < quads ? c : 0)];
+      v[i].x += d.x; v[i].y += d.y; v[i].z += d.z; v[i].w += d.w;
+    }
+  }
+  float partial = 0.f;
+#pragma unroll
+  for (int i = 0; i < QPL; ++i) {
+    int c = lane + i * 64;
+    float4 b = b4[c < quads ? c : 0];
+    v[i].x += b.x; v[i].y += b.y; v[i].z += b.z; v[i].w += b.w;
+    if (c < quads) {
+      if (write_back) xr[c] = v[i];
+      partial += (kind == 0) ? (v[i].x + v[i].y + v[i].z + v[i].w)
+                             : (v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w);
+    }
+  }
+  if (out == nullptr) return;
+  float total = wave_sum(partial);
+  float mean = 0.f, rstd;
+  if (kind == 0) {
+    mean = total / (float)width;
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < QPL; ++i) {
+      if (lane + i * 64 < quads) {
+        float a0 = v[i].x - mean, a1 = v[i].y - mean, a2 = v[i].z - mean, a3 = v[i].w - mean;
+        sq += a0 * a0 + a1 * a1 + a2 * a2 + a3 * a3;
+      }
+    }
+    rstd = 1.0f / sqrtf(wave_sum(sq) / (float)width + eps);
+  } else {
+    rstd = 1.0f / sqrtf(total / (float)width + eps);
+  }
+  T* orow = out + (int64_t)r * width;
+#pragma unroll
+  for (int i = 0; i < QPL; ++i) {
+    int c = lane + i * 64;
+    if (c < quads) {
+      float4 g = g4[c], be = be4[c];
+      float y[4] = {(v[i].x - mean) * rstd * g.x + be.x, (v[i].y - mean) * rstd * g.y + be.y,
+                    (v[i].z - mean) * rstd * g.z + be.z, (v[i].w - mean) * rstd * g.w + be.w};
+      store4<T>(orow + 4 * c, y, 4, true);
+    }
+  }
+}
+
 template <typename T, int VPT>
 static bool launch_add_norm_vec(hipStream_t stream, dim3 grid, float* x, const float* delta, int n_delta,
                                 int64_t delta_stride, const float* bias, const float* gamma, const float* beta,
@@ -206,6 +284,17 @@ static void launch_add_norm(hipStream_t stream, float* x, const float* delta, in
   bool vec = width % 4 == 0 && width <= 4096 && delta_stride % 4 == 0 && aligned(x) && aligned(delta) &&
              aligned(bias) && aligned(gamma) && aligned(beta) && aligned(out);
   bool done = false;
+  if (vec && n_rows >= 512) {        // many rows: a wave per row
+    dim3 row_grid((n_rows + 3) / 4);
+#define BT_ADD_NORM_ROWS(QPL)                                                                                   \
+  hipLaunchKernelGGL((add_norm_rows_kernel<T, QPL>), row_grid, dim3(256), 0, stream, x, delta, n_delta,          \
+                     delta_stride, bias, gamma, beta, eps, kind, out, rows, n_rows, width, write_back)
+    if (width <= 1024) BT_ADD_NORM_ROWS(4);
+    else if (width <= 2048) BT_ADD_NORM_ROWS(8);
+    else BT_ADD_NORM_ROWS(16);
+#undef BT_ADD_NORM_ROWS
+    return;
+  }
   if (vec && width <= 1024)
     done = launch_add_norm_vec<T, 1>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
   else if (vec && width <= 2048)

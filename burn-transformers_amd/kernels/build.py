@@ -38,11 +38,13 @@ def module_source(name):
         return "attention_bf16.hip", [f"-DBT_HEAD_DIM={size}"]
     if name in ("core", "gemm_bf16"):
         return name + ".hip", []
+    if name == "gemm_library":      # host code around hipBLASLt, which it opens at run time
+        return name + ".hip", ["-ldl"]
     raise ValueError(f"unknown kernel module {name!r}")
 
 
 def all_modules():
-    return ["core", "gemm_bf16"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
+    return ["core", "gemm_bf16", "gemm_library"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
 
 
 def _hash(name):
@@ -101,7 +103,9 @@ def compile_module(name, verbose=True):
         raise RuntimeError(f"no writable folder for compiled kernels among {lib_dirs()}")
     lib = os.path.join(target_dir, name + ".so")
     partial = os.path.join(target_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.so")
-    command = [hipcc()] + FLAGS + defs + ["-o", partial, os.path.join(CSRC_DIR, source)]
+    options = [d for d in defs if not d.startswith("-l")]
+    libraries = [d for d in defs if d.startswith("-l")]
+    command = [hipcc()] + FLAGS + options + ["-o", partial, os.path.join(CSRC_DIR, source)] + libraries
     if verbose:
         print(f"[burn_transformers_amd] compiling {name} for {ARCH} ...", file=sys.stderr, flush=True)
     started = time.time()

@@ -6,6 +6,8 @@ that a kernel does not take raises :class:`KernelError` with the kernel's own me
 """
 
 import ctypes
+import os
+import sys
 import threading
 
 import torch  # imported first: the kernel libraries bind to the HIP runtime torch has loaded
@@ -93,8 +95,73 @@ def prepare(dtype, head_dims=()):
     _module("core")
     if dtype == torch.bfloat16:
         _module("gemm_bf16")
+        library_products()
         for size in head_dims:
             _module(f"attention_bf16_hd{size}")
+
+
+# --- the vendor's GEMM library for steps with many rows ---------------------------------------
+
+_library_state = {"tried": False, "lib": None}
+PRODUCTS_ENV = "BURN_TRANSFORMERS_AMD_PRODUCTS"     # "own": never use the vendor's GEMM library
+
+
+def library_products():
+    """The module that runs prompt-sized bfloat16 products through hipBLASLt, or None.
+
+    The reference leaves its matrix products to its backend's library (src/attention.rs:481-513
+    and the feed-forward call ``linear``); here the vendor's library takes the products of steps
+    with more than 64 rows, where it is about 1.6 times as fast as the tile kernel of this
+    package at GPT-2 XL sizes, and the hand-written kernels keep everything else.  The library is
+    opened from the copy that came with torch's HIP runtime and checked once against the tile
+    kernel; if it cannot be opened, or disagrees, the tile kernel does those products too, and
+    a line on stderr says so.
+    """
+    state = _library_state
+    if state["tried"]:
+        return state["lib"]
+    state["tried"] = True
+    if os.environ.get(PRODUCTS_ENV, "") == "own":
+        return None
+    try:
+        lib = _module("gemm_library")
+        candidates = [os.path.join(os.path.dirname(torch.__file__), "lib", "libhipblaslt.so"), "libhipblaslt.so"]
+        version, errors = ctypes.c_int(0), []
+        for path in candidates:
+            if lib.bt_gemm_library_open(path.encode(), ctypes.byref(version)) == 0:
+                break
+            errors.append(lib.bt_last_error().decode())
+        else:
+            raise RuntimeError("; ".join(errors))
+        state["lib"] = lib
+        _check_library_products()
+    except Exception as error:   # the library is an optimisation: without it the own kernels run
+        state["lib"] = None
+        print(f"[burn_transformers_amd] hipBLASLt is not used ({error}); the tile kernel takes its products",
+              file=sys.stderr, flush=True)
+    return state["lib"]
+
+
+def _check_library_products():
+    """One small product with each epilogue the library is given, against the tile kernel."""
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    m, n, k = 96, 80, 64
+    a = torch.randn(m, k, generator=gen, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=gen, device="cuda") / 8).to(torch.bfloat16)
+    bias = torch.randn(n, generator=gen, device="cuda")
+    for make, dtype in ((epilogue_store, torch.bfloat16), (lambda o, b: epilogue_act(o, "gelu_tanh", b), torch.bfloat16),
+                        (epilogue_residual, torch.float32)):
+        mine = torch.ones(m, n, dtype=dtype, device="cuda")
+        theirs = torch.ones(m, n, dtype=dtype, device="cuda")
+        gemm(a, w, make(mine, bias), impl="tile")
+        gemm(a, w, make(theirs, bias), impl="library")
+        error = float((mine.float() - theirs.float()).abs().max())
+        if not error < 0.05:
+            raise RuntimeError(f"its result differs from the tile kernel's by {error}")
+
+
+def _library_takes(epilogue):
+    return epilogue.mode in (EPI_STORE, EPI_RESIDUAL) or (epilogue.mode == EPI_ACT and epilogue.act == 0)
 
 
 # --- epilogues -------------------------------------------------------------------------------
@@ -159,8 +226,9 @@ def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None,
 def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
     """C = a . w^T handed to ``epilogue``.  a: [M, K] (rows may be strided), w: [N, K] contiguous.
 
-    impl: "auto" (float32 -> plain; bfloat16 -> skinny up to 64 rows, else tile), or one of
-    "plain", "tile", "skinny" to force a kernel.  variant picks one of the tile kernel's forms
+    impl: "auto" (float32 -> plain; bfloat16 -> skinny up to 64 rows, beyond that the vendor's
+    library where it is usable and has the epilogue, else tile), or one of "plain", "tile",
+    "skinny", "library" to force one.  variant picks one of the tile kernel's forms
     (0: the fastest the operands allow, 1: any K, 2: lean, 3: direct to LDS).
     """
     m, k = a.shape
@@ -169,7 +237,12 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
         raise KernelError(f"gemm: operands [{m},{k}] {a.dtype} and [{n},{w.shape[1]}] {w.dtype} do not fit")
     dtype = DTYPE_CODES[a.dtype]
     if impl == "auto":
-        impl = "plain" if dtype == FLOAT32 else ("skinny" if m <= 64 else "tile")
+        if dtype == FLOAT32:
+            impl = "plain"
+        elif m <= 64:
+            impl = "skinny"
+        else:
+            impl = "library" if splits == 1 and _library_takes(epilogue) and library_products() else "tile"
     args = (_c_ptr(a.data_ptr()), _c_i64(a.stride(0)), _c_ptr(w.data_ptr()), _c_int(m), _c_int(n), _c_int(k),
             ctypes.byref(epilogue))
     if impl == "plain":
@@ -180,6 +253,14 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
         return
     if dtype != BFLOAT16:
         raise KernelError(f"gemm: the {impl} kernel takes bfloat16 only")
+    if impl == "library":
+        lib = _library_state["lib"] or library_products()
+        if lib is None:
+            raise KernelError("gemm: the vendor's GEMM library is not available")
+        if splits != 1:
+            raise KernelError("gemm: the library product does not split K")
+        _check(lib, lib.bt_gemm_library_bf16(_c_ptr(_stream()), *args))
+        return
     lib = _module("gemm_bf16")
     if impl == "tile":
         _check(lib, lib.bt_gemm_tile_bf16(_c_ptr(_stream()), *args, _c_int(splits), _c_int(variant)))

@@ -52,11 +52,20 @@ class CausalSelfAttention(Mixer):
     def forward(self, h, step, memory, stream):
         tokens = h.shape[0]
         kv = memory.kv()
-        q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
-        if memory.writes:
+        if memory.writes and tokens > 64 and step.dtype_is_bf16 and K.library_products():
+            # a prompt: the vendor's library makes the whole projection, then keys and values are
+            # copied into the cache; the queries are read where they lie
+            qkv = step.buffer("attention.qkv", tokens, self.n_q + 2 * self.n_kv, step.dtype)
+            K.gemm(h, self.qkv_weight, K.epilogue_store(qkv, self.qkv_bias))
+            K.kv_copy(qkv[:, self.n_q:self.n_q + self.n_kv], qkv[:, self.n_q + self.n_kv:], step.tok_seq,
+                      step.tok_pos, kv, to_cache=True)
+            q = qkv[:, :self.n_q]
+        elif memory.writes:
+            q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
             K.gemm(h, self.qkv_weight,
                    K.epilogue_qkv(q, self.n_q, self.n_kv, kv, step.tok_seq, step.tok_pos, self.qkv_bias))
         else:   # the keys and values of another layer are read; only the queries are projected
+            q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
             bias = self.qkv_bias[:self.n_q] if self.qkv_bias is not None else None
             K.gemm(h, self.qkv_weight[:self.n_q], K.epilogue_store(q, bias))
         mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)

@@ -41,6 +41,27 @@ def test_each_request_alone_and_whole(name, dtype, lengths):
     engine.cache.ledger.check()
 
 
+@pytest.mark.parametrize("name,lengths", [("A", [100, 66]), ("B", [150])])
+def test_prompts_without_the_vendor_library(name, lengths, monkeypatch):
+    """Prompts of more than 64 tokens on the package's own tile kernel and fused cache scatter."""
+    from burn_transformers_amd.kernels import library as K
+    monkeypatch.setitem(K._library_state, "tried", True)
+    monkeypatch.setitem(K._library_state, "lib", None)
+    engine = engine_for(name, "bfloat16")
+    prompts = prompts_for(name, lengths, seed=5)
+    slots = [engine.open() for _ in prompts]
+    logits = engine.step(list(zip(slots, prompts)), want=[list(range(len(p))) for p in prompts])
+    begin = 0
+    for ids in prompts:
+        check(logits[begin:begin + len(ids)], plain_logits(name, ids), "bfloat16", f"{name} own kernels {len(ids)}")
+        begin += len(ids)
+    step = engine.step([(slot, [7]) for slot in slots])      # the cache the scatter filled is read
+    for row, ids in enumerate(prompts):
+        check(step[row:row + 1], plain_logits(name, ids + [7])[-1:], "bfloat16", f"{name} own kernels, next token")
+    for slot in slots:
+        engine.close(slot)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,length", [("A", 100), ("B", 150), ("B", 33)])
 def test_last_32_tokens_one_by_one(name, dtype, length):
@@ -134,9 +155,9 @@ def test_unequal_batches_one_after_another(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,count", [("A", 16), ("B", 17), ("A", 40), ("B", 64)])
+@pytest.mark.parametrize("name,count", [("A", 16), ("B", 17), ("A", 40), ("B", 64), ("A", 70)])
 def test_wide_decode_batches(name, dtype, count):
-    """Decode steps of 16, 17..64 sequences take other kernels than small batches do."""
+    """Decode steps of 16, 17..64 and more than 64 sequences take other kernels than small batches do."""
     engine = engine_for(name, dtype, max_tokens=64 * count)
     lengths = [3 + (7 * i) % 20 for i in range(count)]
     requests = prompts_for(name, [n + 3 for n in lengths], seed=70)

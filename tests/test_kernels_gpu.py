@@ -73,6 +73,33 @@ def test_tile_gemm_forms_agree(variant, m, n, k):
                    variant=variant)
 
 
+@pytest.mark.parametrize("m,n,k", [(65, 48, 72), (200, 300, 136), (300, 517, 1600), (2048, 1600, 320)])
+def test_vendor_library_products(m, n, k):
+    """Prompt-sized products through hipBLASLt with the three epilogues it is given, against float64."""
+    if K.library_products() is None:
+        pytest.skip("hipBLASLt could not be opened; the tile kernel takes these products")
+    a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=m, lda=k + 8)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K.gemm(a, w, K.epilogue_store(out, bias), impl="library")
+    assert rel_err(out, want + bias.cpu().double()) < 6e-3
+    K.gemm(a, w, K.epilogue_store(out), impl="library")
+    assert rel_err(out, want) < 6e-3
+    K.gemm(a, w, K.epilogue_act(out, "gelu_tanh", bias), impl="library")
+    assert rel_err(out, gelu_tanh(want + bias.cpu().double())) < 6e-3
+    gen = torch.Generator().manual_seed(1)
+    x0 = torch.randn(m, n, generator=gen)
+    x = x0.clone().to(DEV)
+    K.gemm(a, w, K.epilogue_residual(x, bias), impl="library")
+    assert rel_err(x, x0.double() + want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
+    with pytest.raises(K.KernelError, match="not one the library has"):
+        K.gemm(a, w, K.epilogue_act(out, "gelu_erf", bias), impl="library")
+    # what "auto" picks for these rows gives the same
+    auto = torch.empty_like(out)
+    K.gemm(a, w, K.epilogue_act(out, "gelu_tanh", bias), impl="library")
+    K.gemm(a, w, K.epilogue_act(auto, "gelu_tanh", bias))
+    assert torch.equal(auto, out)
+
+
 @pytest.mark.parametrize("m,n,k,splits", [(1, 100, 136, 1), (8, 4800, 1600, 2), (16, 1600, 1600, 4),
                                           (7, 333, 6400, 8), (3, 50, 1760, 1), (16, 517, 1608, 3),
                                           (2, 16, 8, 1), (9, 40, 3400, 1)])
@@ -218,8 +245,10 @@ def test_attention_finds_one_far_key_among_hundreds():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("width,rows", [(64, 3), (96, 17), (1600, 5), (50, 2)])
+@pytest.mark.parametrize("width,rows", [(64, 3), (96, 17), (1600, 5), (50, 2), (1600, 515), (96, 1030),
+                                        (2052, 513), (4096, 512), (50, 600)])
 def test_add_norm(dtype, width, rows):
+    """Few rows: a work-group per row; 512 rows and more: a wave per row."""
     dt = DTYPES[dtype]
     gen = torch.Generator().manual_seed(width)
     x = (torch.randn(rows, width, generator=gen) * 2 + 0.5).to(DEV)
@@ -242,6 +271,12 @@ def test_add_norm(dtype, width, rows):
     K.add_norm(xs, out, gamma, beta, 1e-3, "layer_norm", delta=delta, bias=bias, rows=pick, write_back=False)
     assert rel_err(out, want[[rows - 1, 0]]) < tol
     assert torch.equal(xs, x)
+    if rows >= 512:     # many selected rows, in another order
+        pick = torch.arange(rows - 1, -1, -1, dtype=torch.int32, device=DEV)
+        out = torch.empty(rows, width, dtype=dt, device=DEV)
+        K.add_norm(xs, out, gamma, beta, 1e-3, "layer_norm", delta=delta, bias=bias, rows=pick, write_back=False)
+        assert rel_err(out, want.flip(0)) < tol
+        assert torch.equal(xs, x)
     # root-mean-square norm, no shift
     xs = x.clone()
     out = torch.empty(rows, width, dtype=dt, device=DEV)

@@ -65,12 +65,22 @@ __device__ __forceinline__ void load_tile(TileOperands& t, const bf16_t* __restr
   }
 }
 
+// The running maximum of a query may lag behind the true one by up to this many powers of two
+// before the sums are rescaled: probabilities then reach at most 2^RESCALE_SLACK instead of 1,
+// which 32-bit sums and bfloat16 operands (a relative format) carry as well, and the rescaling
+// of every output register, three instructions each, is skipped for nearly all tiles.
+#define RESCALE_SLACK 8.0f
+
 // One tile of 32 keys starting at position kb against NQ tiles of 16 queries.
 //   qpos[nq]: position of the query in column lane % 16 of tile nq, -1 if there is none.
 //   valid_end: positions >= valid_end hold no token (their values are replaced by zero).
-template <int NQ>
+//   c: the score scale times log2(e), positive; m[] is kept in those units (powers of two).
+//   MASKED = false is for tiles every query of the wave sees whole (all keys at or before the
+//   first query's position, no window): nothing is compared or replaced there.  Columns without
+//   a query then hold numbers nobody reads.
+template <int NQ, bool MASKED>
 __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, int valid_end,
-                                            const int (&qpos)[NQ], int window, float scale,
+                                            const int (&qpos)[NQ], int window, float c,
                                             const bf16x8 (&q)[NQ][NKS], floatx4 (&o)[NQ][ND],
                                             float (&m)[NQ], float (&l)[NQ]) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
@@ -86,43 +96,56 @@ __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, in
       s[nq][t] = acc;
     }
   }
+  float m_new[NQ];
+  bool behind = false;
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    if (MASKED) {
+      const int qp = qpos[nq];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          int kp = kb + 16 * t + 4 * g + r;
+          bool seen = kp <= qp && (window == 0 || kp > qp - window);
+          s[nq][t][r] = seen ? s[nq][t][r] : -INFINITY;
+        }
+    }
+    float tile_max = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
+                           fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    m_new[nq] = fmaxf(m[nq], tile_max * c);
+    behind = behind || m_new[nq] > m[nq] + RESCALE_SLACK;   // true for the first tile: m starts at -inf
+  }
+  if (__builtin_amdgcn_ballot_w64(behind) != 0) {   // the same for the whole wave: a scalar branch
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      float alpha = m_new[nq] == -INFINITY ? 1.f : exp2f(m[nq] - m_new[nq]);
+      m[nq] = m_new[nq];
+      l[nq] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[nq][dt][r] *= alpha;
+    }
+  }
   bf16x8 pop[NQ];
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
-    const int qp = qpos[nq];
-    float tile_max = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        int kp = kb + 16 * t + 4 * g + r;
-        bool seen = kp <= qp && (window == 0 || kp > qp - window);
-        float v = seen ? s[nq][t][r] * scale : -INFINITY;
-        s[nq][t][r] = v;
-        tile_max = fmaxf(tile_max, v);
-      }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-    float m_new = fmaxf(m[nq], tile_max);
-    float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    float alpha = __expf(m[nq] - m_safe);
+    const float m_use = m[nq] == -INFINITY ? 0.f : m[nq];
     float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float p = __expf(s[nq][t][r] - m_safe);
+        float p = __builtin_amdgcn_exp2f(fmaf(s[nq][t][r], c, -m_use));
         psum += p;
         pop[nq][4 * t + r] = (bf16_t)p;
       }
-    l[nq] = l[nq] * alpha + psum;  // per-lane part of the sum; the four lanes of a column meet at the end
-    m[nq] = m_new;
-#pragma unroll
-    for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) o[nq][dt][r] *= alpha;
+    l[nq] += psum;  // per-lane part of the sum; the four lanes of a column meet at the end
   }
-  const bool ragged = kb + 32 > valid_end;
+  const bool ragged = MASKED && kb + 32 > valid_end;
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt) {
     bf16x4 v0 = tile.v[dt][0], v1 = tile.v[dt][1];
@@ -140,23 +163,64 @@ __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, in
   }
 }
 
+#define LOG2_E 1.4426950408889634f
+
 // Start of the (block, kv head) plane that holds position kb of a sequence.
 __device__ __forceinline__ int64_t tile_plane(const AttnArgs& a, int seq, int kv_head, int kb) {
   int block = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + kb / BT_KV_BLOCK];
   return ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
 }
 
+#ifndef PREFILL_NQ
 #define PREFILL_NQ 2
+#endif
 #define PREFILL_QUERIES_PER_WAVE (16 * PREFILL_NQ)
 #define PREFILL_WAVES 4
 #define PREFILL_QUERIES (PREFILL_QUERIES_PER_WAVE * PREFILL_WAVES)
 
-__global__ void __launch_bounds__(PREFILL_WAVES * 64)
+// Heads up to 64 fit two waves on a SIMD, so that two work-groups share a compute unit; larger
+// heads would spill under that limit and are left one wave.
+#if BT_HEAD_DIM <= 64
+#define PREFILL_OCCUPANCY __attribute__((amdgpu_waves_per_eu(2)))
+#else
+#define PREFILL_OCCUPANCY
+#endif
+
+template <bool PAIRED>
+__global__ void __launch_bounds__((PAIRED ? 2 : 1) * PREFILL_WAVES * 64) PREFILL_OCCUPANCY
 attention_prefill_kernel(AttnArgs a) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i16 = lane & 15, g = lane >> 4;
-  const int seq = blockIdx.z, head = blockIdx.y;
-  const int q_tile = gridDim.x - 1 - blockIdx.x;  // the longest rows of the causal triangle first
-  const int kv_head = head / (a.q_heads / a.kv.kv_heads);
+  // the wave's number is the same in all its lanes; saying so makes the walk over the keys scalar:
+  // the block table is then read through the scalar cache and tests on the position are scalar
+  // branches, neither of which waits for the tiles that are in flight
+  const int lane = threadIdx.x & 63;
+  int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i16 = lane & 15, g = lane >> 4;
+  // Work-groups go to the eight XCDs round-robin by their number, and each XCD has an L2 of its
+  // own.  All work-groups that read one (sequence, key/value head), every query tile of every
+  // query head that shares it, are therefore numbered so that they land on ONE XCD: its keys and
+  // values come from memory once and from that L2 afterwards (spread over all eight, the keys and
+  // values of a step were read from memory eight times over, and that set the kernel's time).
+  //
+  // PAIRED: a work-group is two query tiles of 128, four waves each: tile i from the end of the
+  // causal triangle and tile i from its start.  A query at position p walks p / 32 tiles of keys,
+  // so every SIMD of a compute unit gets one long and one short wave and all finish together;
+  // with a work-group per tile, the units that drew two late tiles set the kernel's time.  It is
+  // used when there are more tiles than compute units (otherwise a work-group per tile spreads
+  // the work further) and for heads up to 64 (eight waves leave each 256 registers).
+  const int group = a.q_heads / a.kv.kv_heads;
+  const int q_tiles = (a.max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES;
+  const int pairs = PAIRED ? (q_tiles + 1) / 2 : q_tiles;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int unit = (slot / (group * pairs)) * 8 + xcd;      // which (sequence, key/value head)
+  if (unit >= a.n_seqs * a.kv.kv_heads) return;
+  const int within = slot % (group * pairs);
+  const int seq = unit / a.kv.kv_heads, kv_head = unit % a.kv.kv_heads;
+  const int head = kv_head * group + within % group;
+  const int pair = within / group, late = q_tiles - 1 - pair;
+  const bool second = PAIRED && wave >= PREFILL_WAVES;   // the wave belongs to the early tile of the pair
+  if (second && pair == late) return;                    // an odd number of tiles: the middle one is alone
+  const int q_tile = second ? pair : late;
+  wave &= PREFILL_WAVES - 1;
   const int off = a.seq_off[seq], count = a.seq_off[seq + 1] - off, start = a.seq_start[seq];
   const int q0 = q_tile * PREFILL_QUERIES + wave * PREFILL_QUERIES_PER_WAVE;
   if (q0 >= count) return;
@@ -190,18 +254,33 @@ attention_prefill_kernel(AttnArgs a) {
   const int valid_end = start + count;
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
-  TileOperands current, next;
-  if (lo < hi) {
-    int64_t plane = tile_plane(a, seq, kv_head, lo);
-    load_tile(next, keys + plane, values + plane, lo);
-  }
-  for (int kb = lo; kb < hi; kb += 32) {
-    current = next;
-    if (kb + 32 < hi) {
-      int64_t plane = tile_plane(a, seq, kv_head, kb + 32);
-      load_tile(next, keys + plane, values + plane, kb + 32);
-    }
-    attend_tile<PREFILL_NQ>(current, kb, valid_end, qpos, a.window, a.scale, q, o, m, l);
+  // The tiles alternate between two sets of registers, each named at compile time, so nothing
+  // is copied: while one is multiplied the other is in flight.  (A third set, two tiles ahead,
+  // costs the registers that let two work-groups share a compute unit, and measured slower.)
+  const float c = a.scale * LOG2_E;
+  const int whole_until = a.window == 0 ? start + q0 + 1 : 0;   // tiles ending here or before are seen whole
+  // A fetch beyond the last tile reads the first one again instead of being skipped: with the same
+  // number of loads in flight on every path, the wait before a tile is for that tile only.
+  TileOperands t0, t1;
+  auto fetch = [&](TileOperands& into, int kb) {
+    const int kf = kb < hi ? kb : lo;
+    int64_t plane = tile_plane(a, seq, kv_head, kf);
+    load_tile(into, keys + plane, values + plane, kf);
+  };
+  auto attend = [&](const TileOperands& tile, int kb) {
+    if (kb + 32 <= whole_until)
+      attend_tile<PREFILL_NQ, false>(tile, kb, valid_end, qpos, a.window, c, q, o, m, l);
+    else
+      attend_tile<PREFILL_NQ, true>(tile, kb, valid_end, qpos, a.window, c, q, o, m, l);
+  };
+  if (lo >= hi) return;   // (cannot happen: a wave with a query sees at least that query's key)
+  fetch(t0, lo);
+  fetch(t1, lo + 32);
+  for (int kb = lo; kb < hi; kb += 64) {
+    attend(t0, kb);
+    fetch(t0, kb + 64);
+    if (kb + 32 < hi) attend(t1, kb + 32);
+    fetch(t1, kb + 96);
   }
   bf16_t* out = static_cast<bf16_t*>(a.out);
 #pragma unroll
@@ -227,7 +306,9 @@ __global__ void __launch_bounds__(DECODE_WAVES * 64)
 attention_decode_kernel(AttnArgs a) {
   // per wave: maximum and sum of each query column, and its output row; `group` columns are real
   extern __shared__ float sm[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i16 = lane & 15, g = lane >> 4;
+  // (the wave's number is said to be the same in all lanes, so that tests on it are scalar branches)
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i16 = lane & 15, g = lane >> 4;
   const int seq = blockIdx.y, kv_head = blockIdx.x;
   const int group = a.q_heads / a.kv.kv_heads;
   float* sm_m = sm;                                   // [DECODE_WAVES][group]
@@ -274,19 +355,23 @@ attention_decode_kernel(AttnArgs a) {
     int block = (a.window == 0 && j < 2) ? (j == 0 ? early_block0 : early_block1) : block_row[kb / BT_KV_BLOCK];
     return ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
   };
+  const float c = a.scale * LOG2_E;
+  auto fetch = [&](TileOperands& into, int kb, int j) {
+    if (kb <= pos) {
+      int64_t plane = plane_of(kb, j);
+      load_tile(into, keys + plane, values + plane, kb);
+    }
+  };
+  auto attend = [&](const TileOperands& tile, int kb) {   // one form: this kernel waits for memory, not for the ALU
+    attend_tile<1, true>(tile, kb, pos + 1, qpos, a.window, c, q, o, m, l);
+  };
   TileOperands current, next;
-  if (first <= pos) {
-    int64_t plane = plane_of(first, 0);
-    load_tile(next, keys + plane, values + plane, first);
-  }
+  fetch(next, first, 0);
   int j = 0;
   for (int kb = first; kb <= pos; kb += stride, ++j) {
     current = next;
-    if (kb + stride <= pos) {
-      int64_t plane = plane_of(kb + stride, j + 1);
-      load_tile(next, keys + plane, values + plane, kb + stride);
-    }
-    attend_tile<1>(current, kb, pos + 1, qpos, a.window, a.scale, q, o, m, l);
+    fetch(next, kb + stride, j + 1);
+    attend(current, kb);
   }
   float total = l[0];
   total += __shfl_xor(total, 16, 64);
@@ -312,7 +397,7 @@ attention_decode_kernel(AttnArgs a) {
     if (top != -INFINITY) {
 #pragma unroll
       for (int w = 0; w < DECODE_WAVES; ++w) {
-        float f = __expf(sm_m[w * group + j] - top);
+        float f = exp2f(sm_m[w * group + j] - top);   // the maxima are kept in powers of two
         num += sm_o[(w * group + j) * HD + channel] * f;
         den += sm_l[w * group + j] * f;
       }
@@ -326,6 +411,7 @@ static int check_args(const AttnArgs& a, const char* who) {
   if (a.kv.kv_heads <= 0 || a.q_heads <= 0 || a.q_heads % a.kv.kv_heads != 0)
     BT_REFUSE("%s: %d query heads cannot share %d key/value heads", who, a.q_heads, a.kv.kv_heads);
   if (a.window < 0) BT_REFUSE("%s: window %d must not be negative", who, a.window);
+  if (!(a.scale > 0.f)) BT_REFUSE("%s: the score scale %g must be positive (the maximum is taken before scaling)", who, a.scale);
   if (!a.q || !a.out || !a.seq_off || !a.seq_start || !a.kv.blocks || !a.kv.keys || !a.kv.values)
     BT_REFUSE("%s: missing operand", who);
   if (a.ldq % 8 != 0 || a.ldo % 4 != 0 || ((uintptr_t)a.q & 15) || ((uintptr_t)a.out & 7))
@@ -340,8 +426,28 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
   int rc = check_args(*args, "attention_prefill_bf16");
   if (rc) return rc;
   if (args->max_count <= 0) BT_REFUSE("attention_prefill_bf16: max_count %d must be positive", args->max_count);
-  dim3 grid((args->max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES, args->q_heads, args->n_seqs);
-  hipLaunchKernelGGL(attention_prefill_kernel, grid, dim3(PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);
+  const int q_tiles = (args->max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES;
+  const int group = args->q_heads / args->kv.kv_heads;
+  const int64_t units = (int64_t)args->n_seqs * args->kv.kv_heads;
+  const int64_t units_per_xcd = (units + 7) / 8;
+  static int compute_units = 0;
+  if (compute_units == 0) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+      compute_units = 256;
+  }
+  const bool paired = HD <= 64 && units * group * q_tiles > compute_units;
+  const int64_t groups = 8 * units_per_xcd * group * (paired ? (q_tiles + 1) / 2 : q_tiles);
+  if (groups > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: %lld work-groups are too many", (long long)groups);
+  dim3 grid((unsigned)groups);
+  if constexpr (HD <= 64) {   // (the paired form is not even built for larger heads)
+    if (paired) {
+      hipLaunchKernelGGL(attention_prefill_kernel<true>, grid, dim3(2 * PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);
+      return bt_check_launch("attention_prefill_bf16");
+    }
+  }
+  hipLaunchKernelGGL(attention_prefill_kernel<false>, grid, dim3(PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);
   return bt_check_launch("attention_prefill_bf16");
 }
 

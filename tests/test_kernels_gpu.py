@@ -203,7 +203,18 @@ def test_attention_plain(dtype, q_heads, kv_heads, hd, totals, counts, window):
     assert rel_err(out, want) < (3e-6 if dtype == "float32" else 8e-3)
 
 
-@pytest.mark.parametrize("q_heads,kv_heads,hd,totals,counts,window", ATTN_CASES)
+# More query tiles than the GPU has compute units: the prefill kernel then pairs a late tile
+# with an early one in each work-group (an even and an odd number of tiles, sequences shorter
+# than the longest, chunks on non-empty caches, a window).
+PAIRED_CASES = [
+    (8, 4, 32, [700, 300, 650, 129, 640, 513], [700, 300, 650, 129, 640, 513], 0),
+    (4, 4, 64, [600] * 13 + [100], [600] * 13 + [100], 0),
+    (8, 4, 32, [900, 800, 700, 650, 600, 560, 520, 512, 1000], [500, 500, 300, 129, 128, 1, 64, 500, 512], 0),
+    (6, 6, 64, [400] * 12, [400] * 12, 100),
+]
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,hd,totals,counts,window", ATTN_CASES + PAIRED_CASES)
 def test_attention_mfma(q_heads, kv_heads, hd, totals, counts, window):
     dt = torch.bfloat16
     case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=3, poison=True)
@@ -242,6 +253,46 @@ def test_attention_finds_one_far_key_among_hundreds():
                                     1, 1, 1, 1.0, 0)
             K.attention(args, dt, decode=decode, impl=impl)
             assert rel_err(out, want) < 1e-2, (target, impl, decode)
+
+
+@pytest.mark.parametrize("pattern", ["ramp", "jumps", "falling"])
+def test_attention_with_scores_that_rise_and_jump(pattern):
+    """The running maximum is allowed to lag a little before sums are rescaled: scores that creep
+    up (never rescaled after the first tile, probabilities above one), jump (rescaled at once)
+    or fall (the first tile dominates) must all give the plain result."""
+    dt = torch.bfloat16
+    hd, total = 64, 600
+    case = PagedCase([total], [total], 1, hd, dt, DEV, seed=11)
+    position = torch.arange(total, dtype=torch.float32)
+    if pattern == "ramp":
+        gain = position / total * 30.0                    # about 1.6 per tile of 32 keys
+    elif pattern == "jumps":
+        gain = (position // 97) * 25.0 + (position % 7)
+    else:
+        gain = 40.0 - position / total * 40.0
+    case.k_rows[0][:] *= 0.05
+    case.k_rows[0][:, 5] = gain.to(dt)
+    seq = torch.zeros(total, dtype=torch.int32, device=DEV)
+    pos = torch.arange(total, dtype=torch.int32, device=DEV)
+    K.kv_copy(case.k_rows[0].to(DEV), case.v_rows[0].to(DEV), seq, pos, case.view(), True)
+    gen = torch.Generator().manual_seed(12)
+    q = torch.randn(total, hd, generator=gen) * 0.1
+    q[:, 5] = 1.0
+    q = q.to(dt).to(DEV)
+    want = case.reference(q, 1, 1.0)
+    out = torch.empty(total, hd, dtype=dt, device=DEV)
+    args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                            1, 1, total, 1.0, 0)
+    K.attention(args, dt, decode=False, impl="mfma")
+    assert rel_err(out, want) < 1.2e-2
+    # the last query alone, through the decode kernel (its waves meet with their own maxima)
+    one = PagedCase([total], [1], 1, hd, dt, DEV, seed=11)
+    K.kv_copy(case.k_rows[0].to(DEV), case.v_rows[0].to(DEV), seq, pos, one.view(), True)
+    out1 = torch.empty(1, hd, dtype=dt, device=DEV)
+    args = K.attention_args(q[-1:], out1, one.view(), one.tok_seq, one.tok_pos, one.seq_off, one.seq_start,
+                            1, 1, 1, 1.0, 0)
+    K.attention(args, dt, decode=True, impl="mfma")
+    assert rel_err(out1, want[-1:]) < 1.2e-2
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

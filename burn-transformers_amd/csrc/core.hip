@@ -523,12 +523,60 @@ __global__ void kv_copy_kernel(T* __restrict__ k_rows, T* __restrict__ v_rows, i
   }
 }
 
+// The same into the cache for bfloat16 rows of a prompt, with wide accesses.  Values lie with
+// four consecutive positions interleaved per channel, so the work-group of the FIRST token of
+// each run of up to four tokens that share such a group (same sequence, consecutive positions,
+// same position / 4) stores the whole run: a full run is one 8-byte store per channel.  Keys go
+// eight channels (16 bytes) at a time.  Work-groups of the other tokens of a run leave at once.
+__global__ void __launch_bounds__(256)
+kv_store_bf16_kernel(const bf16_t* __restrict__ k_rows, const bf16_t* __restrict__ v_rows, int64_t ld,
+                     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, KvView kv, int tokens) {
+  const int t = blockIdx.x;
+  const int seq = tok_seq[t], pos = tok_pos[t];
+  const bool continues = t > 0 && tok_seq[t - 1] == seq && tok_pos[t - 1] == pos - 1 && (pos & 3) != 0;
+  if (continues) return;
+  int run = 1;
+  while (run < 4 && t + run < tokens && tok_seq[t + run] == seq && tok_pos[t + run] == pos + run &&
+         ((pos + run) & 3) != 0)
+    ++run;
+  const int hd = kv.head_dim, width = kv.kv_heads * hd;
+  bf16_t* keys = static_cast<bf16_t*>(kv.keys);
+  bf16_t* values = static_cast<bf16_t*>(kv.values);
+  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
+  for (int c = threadIdx.x * 8; c < width; c += 256 * 8) {
+    int head = c / hd, channel = c % hd;
+    int64_t base = kv_block_base(kv, seq, pos, head);     // the run lies in one block
+    for (int i = 0; i < run; ++i)
+      *reinterpret_cast<int4v*>(keys + base + key_offset(hd, pos + i, channel)) =
+          *reinterpret_cast<const int4v*>(k_rows + (int64_t)(t + i) * ld + c);
+  }
+  for (int c = threadIdx.x; c < width; c += 256) {
+    int head = c / hd, channel = c % hd;
+    int64_t base = kv_block_base(kv, seq, pos, head);
+    if (run == 4 && (pos & 3) == 0) {
+      bf16x4 quad = {v_rows[(int64_t)t * ld + c], v_rows[(int64_t)(t + 1) * ld + c],
+                     v_rows[(int64_t)(t + 2) * ld + c], v_rows[(int64_t)(t + 3) * ld + c]};
+      *reinterpret_cast<bf16x4*>(values + base + value_offset(hd, pos, channel)) = quad;
+    } else {
+      for (int i = 0; i < run; ++i)
+        values[base + value_offset(hd, pos + i, channel)] = v_rows[(int64_t)(t + i) * ld + c];
+    }
+  }
+}
+
 BT_EXPORT int bt_kv_copy(void* stream, int dtype, void* k_rows, void* v_rows, int64_t ld,
                          const int* tok_seq, const int* tok_pos, const KvView* kv, int tokens,
                          int to_cache) {
   if (tokens <= 0) return BT_OK;
   if (kv->head_dim <= 0 || kv->head_dim % 4 != 0) BT_REFUSE("kv_copy: head size %d must be a multiple of 4", kv->head_dim);
   dim3 grid(tokens), block(256);
+  const bool wide = dtype != 0 && to_cache && tokens > 64 && kv->head_dim % 8 == 0 && ld % 8 == 0 &&
+                    ((uintptr_t)k_rows & 15) == 0 && ((uintptr_t)kv->keys & 15) == 0 && ((uintptr_t)kv->values & 7) == 0;
+  if (wide) {
+    hipLaunchKernelGGL(kv_store_bf16_kernel, grid, block, 0, (hipStream_t)stream, (const bf16_t*)k_rows,
+                       (const bf16_t*)v_rows, ld, tok_seq, tok_pos, *kv, tokens);
+    return bt_check_launch("kv_copy");
+  }
   if (dtype == 0)
     hipLaunchKernelGGL(kv_copy_kernel<float>, grid, block, 0, (hipStream_t)stream, (float*)k_rows,
                        (float*)v_rows, ld, tok_seq, tok_pos, *kv, to_cache);

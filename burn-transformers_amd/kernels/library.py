@@ -215,6 +215,8 @@ def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None,
     else:
         n_delta, stride = 1, 0
     n_rows = rows.numel() if rows is not None else x.shape[0]
+    if delta is None and bias is None:
+        write_back = False      # nothing is added: the stream already holds what would be written
     out_dtype = DTYPE_CODES[out.dtype] if out is not None else FLOAT32
     _check(lib, lib.bt_add_norm(
         _c_ptr(_stream()), _c_int(out_dtype), _c_ptr(x.data_ptr()), _c_ptr(_ptr(delta)), _c_int(n_delta),

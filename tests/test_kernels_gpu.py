@@ -203,6 +203,31 @@ def test_attention_plain(dtype, q_heads, kv_heads, hd, totals, counts, window):
     assert rel_err(out, want) < (3e-6 if dtype == "float32" else 8e-3)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("totals,counts", [([5, 70], [5, 3]), ([130, 67, 9, 260], [130, 66, 2, 77]),
+                                           ([300], [299])])
+def test_kv_copy_round_trip(dtype, totals, counts):
+    """Rows written into the paged cache (a few tokens: element by element; a prompt in bfloat16: runs
+    of four positions at a time, starting anywhere) come back unchanged, and nothing else is touched."""
+    dt = DTYPES[dtype]
+    kv_heads, hd = 3, 16
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=4)
+    before_k, before_v = case.read_back()
+    gen = torch.Generator().manual_seed(8)
+    pitch = 2 * kv_heads * hd + 8
+    rows = torch.randn(case.n_tokens, pitch, generator=gen).to(dt).to(DEV)
+    new_k, new_v = rows[:, :kv_heads * hd], rows[:, kv_heads * hd:2 * kv_heads * hd]
+    K.kv_copy(new_k, new_v, case.tok_seq, case.tok_pos, case.view(), True)
+    after_k, after_v = case.read_back()
+    row, begin = 0, 0
+    for total, count in zip(totals, counts):
+        old = slice(begin, begin + total - count)
+        new = slice(begin + total - count, begin + total)
+        assert torch.equal(after_k[old], before_k[old]) and torch.equal(after_v[old], before_v[old])
+        assert torch.equal(after_k[new], new_k[row:row + count]) and torch.equal(after_v[new], new_v[row:row + count])
+        row, begin = row + count, begin + total
+
+
 # More query tiles than the GPU has compute units: the prefill kernel then pairs a late tile
 # with an early one in each work-group (an even and an odd number of tiles, sequences shorter
 # than the longest, chunks on non-empty caches, a window).

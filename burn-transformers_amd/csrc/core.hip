@@ -523,37 +523,44 @@ __global__ void kv_copy_kernel(T* __restrict__ k_rows, T* __restrict__ v_rows, i
   }
 }
 
-// The same into the cache for bfloat16 rows of a prompt, with wide accesses.  Values lie with
-// four consecutive positions interleaved per channel, so the work-group of the FIRST token of
-// each run of up to four tokens that share such a group (same sequence, consecutive positions,
-// same position / 4) stores the whole run: a full run is one 8-byte store per channel.  Keys go
-// eight channels (16 bytes) at a time.  Work-groups of the other tokens of a run leave at once.
+// The same into the cache for bfloat16 rows of a prompt, with wide accesses.  Every token's
+// work-group copies its own key row, eight channels (16 bytes) at a time.  Values lie with four
+// consecutive positions interleaved per channel, so the work-group of the FIRST token of each run
+// of up to four tokens that share such a group (same sequence, consecutive positions, same
+// position / 4) stores the values of the whole run: a full run is one 8-byte store per channel.
 __global__ void __launch_bounds__(256)
 kv_store_bf16_kernel(const bf16_t* __restrict__ k_rows, const bf16_t* __restrict__ v_rows, int64_t ld,
                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, KvView kv, int tokens) {
   const int t = blockIdx.x;
-  const int seq = tok_seq[t], pos = tok_pos[t];
-  const bool continues = t > 0 && tok_seq[t - 1] == seq && tok_pos[t - 1] == pos - 1 && (pos & 3) != 0;
-  if (continues) return;
-  int run = 1;
-  while (run < 4 && t + run < tokens && tok_seq[t + run] == seq && tok_pos[t + run] == pos + run &&
-         ((pos + run) & 3) != 0)
-    ++run;
+  // the neighbours' sequences and positions, all asked for at once (indices clamped into the step)
+  int seqs[5], poss[5];
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    int u = t - 1 + i;
+    u = u < 0 ? 0 : (u < tokens ? u : tokens - 1);
+    seqs[i] = tok_seq[u];
+    poss[i] = tok_pos[u];
+  }
+  const int seq = seqs[1], pos = poss[1];
   const int hd = kv.head_dim, width = kv.kv_heads * hd;
   bf16_t* keys = static_cast<bf16_t*>(kv.keys);
   bf16_t* values = static_cast<bf16_t*>(kv.values);
   typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
   for (int c = threadIdx.x * 8; c < width; c += 256 * 8) {
     int head = c / hd, channel = c % hd;
-    int64_t base = kv_block_base(kv, seq, pos, head);     // the run lies in one block
-    for (int i = 0; i < run; ++i)
-      *reinterpret_cast<int4v*>(keys + base + key_offset(hd, pos + i, channel)) =
-          *reinterpret_cast<const int4v*>(k_rows + (int64_t)(t + i) * ld + c);
+    *reinterpret_cast<int4v*>(keys + kv_block_base(kv, seq, pos, head) + key_offset(hd, pos, channel)) =
+        *reinterpret_cast<const int4v*>(k_rows + (int64_t)t * ld + c);
   }
+  const bool continues = t > 0 && seqs[0] == seq && poss[0] == pos - 1 && (pos & 3) != 0;
+  if (continues) return;
+  int run = 1;
+#pragma unroll
+  for (int i = 1; i < 4; ++i)
+    if (run == i && t + i < tokens && seqs[1 + i] == seq && poss[1 + i] == pos + i && ((pos + i) & 3) != 0) run = i + 1;
   for (int c = threadIdx.x; c < width; c += 256) {
     int head = c / hd, channel = c % hd;
-    int64_t base = kv_block_base(kv, seq, pos, head);
-    if (run == 4 && (pos & 3) == 0) {
+    int64_t base = kv_block_base(kv, seq, pos, head);     // the run lies in one block
+    if (run == 4) {                                       // then pos is a multiple of four
       bf16x4 quad = {v_rows[(int64_t)t * ld + c], v_rows[(int64_t)(t + 1) * ld + c],
                      v_rows[(int64_t)(t + 2) * ld + c], v_rows[(int64_t)(t + 3) * ld + c]};
       *reinterpret_cast<bf16x4*>(values + base + value_offset(hd, pos, channel)) = quad;

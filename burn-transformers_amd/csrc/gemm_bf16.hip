@@ -436,20 +436,27 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
 // what splitting K is for when there are few output columns, and (b) has ONE round trip to
 // memory on its critical path: everything the epilogue needs (bias, old residual, cache
 // addresses) is fetched together with the first batch of weights, without a branch in between.
-template <int MT, int U, int WAVES>
+// MT row blocks of 16 (activations) by NT column blocks of 16 (weights) per work-group.  With
+// more than 16 rows the activations a work-group reads (all rows, its whole K range) outweigh its
+// weights, and they are read once per work-group: two column blocks halve that traffic.
+template <int MT, int NT, int U, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
                    int K, Epilogue epi) {
-  __shared__ __attribute__((aligned(16))) float red[WAVES][MT][64][4];
+  __shared__ __attribute__((aligned(16))) float red[WAVES][MT * NT][64][4];
+  static_assert(MT * NT <= WAVES, "one wave finishes each block of the work-group's output");
   // the wave's number is the same in all its lanes: saying so keeps every test on it a scalar
   // branch, which costs no wait for loads in flight (a divergent one does)
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int i16 = lane & 15, g = lane >> 4;
-  const int n_base = blockIdx.x * 16;
+  const int n_base = blockIdx.x * 16 * NT;
   const int split = blockIdx.y, splits = gridDim.y;
-  int n = n_base + i16;
-  n = n < N ? n : N - 1;
-  const bf16_t* w_row = W + (int64_t)n * K;
+  const bf16_t* w_row[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    int n = n_base + nt * 16 + i16;
+    w_row[nt] = W + (int64_t)(n < N ? n : N - 1) * K;
+  }
   const bf16_t* a_row[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -465,21 +472,25 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
   typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
   const int chunks = chunks_of(K);
   const int stride = splits * WAVES;
-  floatx4 acc[MT];
+  floatx4 acc[MT][NT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  int4v wv[U], av[U][MT];
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  int4v wv[U][NT], av[U][MT];
   auto issue = [&](int c0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int cc = c0 + u * stride;
-      wv[u] = int4v{0, 0, 0, 0};
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) wv[u][nt] = int4v{0, 0, 0, 0};
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) av[u][mt] = int4v{0, 0, 0, 0};
       if (cc < chunks) {
         int k = cc * 32 + g * 8;
         int kc = k < K ? k : K - 8;
-        wv[u] = *reinterpret_cast<const int4v*>(w_row + kc);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wv[u][nt] = *reinterpret_cast<const int4v*>(w_row[nt] + kc);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + kc);
       }
@@ -489,19 +500,25 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int keep = (c0 + u * stride) * 32 + g * 8 < K ? -1 : 0;
-      bf16x8 w = __builtin_bit_cast(bf16x8, wv[u] & keep);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, __builtin_bit_cast(bf16x8, av[u][mt]), acc[mt], 0, 0, 0);
+      for (int nt = 0; nt < NT; ++nt) {
+        bf16x8 w = __builtin_bit_cast(bf16x8, wv[u][nt] & keep);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, __builtin_bit_cast(bf16x8, av[u][mt]), acc[mt][nt], 0, 0, 0);
+      }
     }
   };
   int c0 = split * WAVES + wave;
   issue(c0);
-  // wave w < MT finishes row block w: lane holds D[i][j], i = 4 * (lane / 16) + r (column n),
-  // j = lane % 16 (row m); what its epilogue needs is fetched now, behind the first batch
-  const int out_m = (wave < MT ? wave : 0) * 16 + i16, out_n0 = n_base + g * 4;
+  // wave w < MT * NT finishes row block w / NT of column block w % NT: lane holds D[i][j],
+  // i = 4 * (lane / 16) + r (column n), j = lane % 16 (row m); what its epilogue needs is
+  // fetched now, behind the first batch
+  const int blocks = MT * NT;
+  const int mine = wave < blocks ? wave : 0;
+  const int out_m = (mine / NT) * 16 + i16, out_n0 = n_base + (mine % NT) * 16 + g * 4;
   EpiloguePrefetch pre = {};
-  if (wave < MT) pre = epilogue_prefetch(epi, M, N, out_m, out_n0, split);
+  if (wave < blocks) pre = epilogue_prefetch(epi, M, N, out_m, out_n0, split);
   multiply(c0);
   for (c0 += stride * U; c0 < chunks; c0 += stride * U) {
     issue(c0);
@@ -509,9 +526,11 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
   }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
-    *reinterpret_cast<floatx4*>(&red[wave][mt][lane][0]) = acc[mt];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      *reinterpret_cast<floatx4*>(&red[wave][mt * NT + nt][lane][0]) = acc[mt][nt];
   __syncthreads();
-  if (wave < MT) {
+  if (wave < blocks) {
     float v[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int w = 0; w < WAVES; ++w)
@@ -593,7 +612,7 @@ BT_EXPORT int bt_gemm_tile_bf16(void* stream, const void* A, int64_t lda, const 
 }
 
 BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                                  const Epilogue* epi, int splits) {
+                                  const Epilogue* epi, int splits, int variant) {
   if (M <= 0) return BT_OK;
   if (M > 64) BT_REFUSE("gemm_skinny_bf16: %d rows, at most 64", M);
   int rc = check_operands("gemm_skinny_bf16", A, lda, W, M, N, K, *epi, splits);
@@ -601,12 +620,16 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  dim3 grid((N + 15) / 16, splits);
+  // variant 1 (measurements and tests): one column block per work-group also beyond 16 rows
   if (M <= 16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, 8, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi);
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 8, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
+  else if (M <= 32 && variant == 1)
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, 1, 4, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
+  else if (variant == 1)
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, 1, 2, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
   else if (M <= 32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 4, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi);
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, 2, 4, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
   else
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi);
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 2, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
   return bt_check_launch("gemm_skinny_bf16");
 }

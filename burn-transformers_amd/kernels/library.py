@@ -231,7 +231,8 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
     impl: "auto" (float32 -> plain; bfloat16 -> skinny up to 64 rows, beyond that the vendor's
     library where it is usable and has the epilogue, else tile), or one of "plain", "tile",
     "skinny", "library" to force one.  variant picks one of the tile kernel's forms
-    (0: the fastest the operands allow, 1: any K, 2: lean, 3: direct to LDS).
+    (0: the fastest the operands allow, 1: any K, 2: lean, 3: direct to LDS) or, for the skinny
+    kernel beyond 16 rows, one column block per work-group (1) instead of two (0).
     """
     m, k = a.shape
     n = w.shape[0]
@@ -267,7 +268,7 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
     if impl == "tile":
         _check(lib, lib.bt_gemm_tile_bf16(_c_ptr(_stream()), *args, _c_int(splits), _c_int(variant)))
     else:
-        _check(lib, lib.bt_gemm_skinny_bf16(_c_ptr(_stream()), *args, _c_int(splits)))
+        _check(lib, lib.bt_gemm_skinny_bf16(_c_ptr(_stream()), *args, _c_int(splits), _c_int(variant)))
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,

@@ -145,8 +145,8 @@ def compute_units(device):
 def split_count(rows, columns, k, units=256):
     """How many ways a residual-writing product splits its K range (up to 64 rows; 1 beyond).
 
-    The skinny product gives one work-group 16 output columns and one slice of K, and its time
-    is set by the compute unit that has to pull the most bytes: a unit takes a work-group of
+    The skinny product gives one work-group 16 output columns (32 beyond 16 rows) and one slice
+    of K, and its time is set by the compute unit that has to pull the most bytes: a unit takes a work-group of
     ``per`` chunks of 32 in about ``per + 10`` units of time (the ten are the work-group's own
     start and its reduction), and ``tiles * splits`` work-groups land on ``units`` compute units
     in whole rounds.  Measured on 100 tiles: K 6400 takes 13.9 / 8.6 / 8.5 / 7.6 / 9.3 us with
@@ -154,7 +154,7 @@ def split_count(rows, columns, k, units=256):
     """
     if rows > 64:
         return 1
-    tiles = (columns + 15) // 16
+    tiles = (columns + 15) // 16 if rows <= 16 else (columns + 31) // 32   # beyond 16 rows: 32 columns each
     chunks = (k + 31) // 32
     best, best_cost = 1, None
     for splits in range(1, 9):

@@ -197,11 +197,16 @@ add_norm_rows_kernel(float* __restrict__ x, const float* __restrict__ delta, int
   const float4* b4 = bias ? reinterpret_cast<const float4*>(bias) : z4;
   const float4* g4 = gamma ? reinterpret_cast<const float4*>(gamma) : z4;
   const float4* be4 = beta ? reinterpret_cast<const float4*>(beta) : z4;
-  float4 v[QPL];
+  // every vector a lane needs is asked for before anything is added: one trip to memory
+  float4 v[QPL], b[QPL], g[QPL], be[QPL];
 #pragma unroll
   for (int i = 0; i < QPL; ++i) {
     int c = lane + i * 64;
-    v[i] = xr[c < quads ? c : 0];
+    int cc = c < quads ? c : 0;
+    v[i] = xr[cc];
+    b[i] = b4[cc];
+    g[i] = g4[cc];
+    be[i] = be4[cc];
   }
   for (int s = 0; s < n_delta; ++s) {          // same order of additions as the plain kernel
 #pragma unroll
@@ -215,8 +220,7 @@ add_norm_rows_kernel(float* __restrict__ x, const float* __restrict__ delta, int
 #pragma unroll
   for (int i = 0; i < QPL; ++i) {
     int c = lane + i * 64;
-    float4 b = b4[c < quads ? c : 0];
-    v[i].x += b.x; v[i].y += b.y; v[i].z += b.z; v[i].w += b.w;
+    v[i].x += b[i].x; v[i].y += b[i].y; v[i].z += b[i].z; v[i].w += b[i].w;
     if (c < quads) {
       if (write_back) xr[c] = v[i];
       partial += (kind == 0) ? (v[i].x + v[i].y + v[i].z + v[i].w)
@@ -245,9 +249,8 @@ add_norm_rows_kernel(float* __restrict__ x, const float* __restrict__ delta, int
   for (int i = 0; i < QPL; ++i) {
     int c = lane + i * 64;
     if (c < quads) {
-      float4 g = g4[c], be = be4[c];
-      float y[4] = {(v[i].x - mean) * rstd * g.x + be.x, (v[i].y - mean) * rstd * g.y + be.y,
-                    (v[i].z - mean) * rstd * g.z + be.z, (v[i].w - mean) * rstd * g.w + be.w};
+      float y[4] = {(v[i].x - mean) * rstd * g[i].x + be[i].x, (v[i].y - mean) * rstd * g[i].y + be[i].y,
+                    (v[i].z - mean) * rstd * g[i].z + be[i].z, (v[i].w - mean) * rstd * g[i].w + be[i].w};
       store4<T>(orow + 4 * c, y, 4, true);
     }
   }

@@ -299,6 +299,249 @@ attention_prefill_kernel(AttnArgs a) {
   }
 }
 
+// A whole block of 64 keys at once, for the kernel that has it in LDS: the same steps as
+// attend_tile with half as many maxima, exchanges between lanes and rescaling tests per key,
+// and four independent score blocks for the scheduler to interleave (one wave is often alone
+// on its SIMD here, so nothing else hides the latency of a dependent chain).
+struct BlockOperands {
+  bf16x8 k[4][NKS];
+  bf16x4 v[ND][4];
+};
+
+template <int NQ, bool MASKED>
+__device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, int valid_end,
+                                             const int (&qpos)[NQ], float c, const bf16x8 (&q)[NQ][NKS],
+                                             floatx4 (&o)[NQ][ND], float (&m)[NQ], float (&l)[NQ]) {
+  const int lane = threadIdx.x & 63, g = lane >> 4;
+  floatx4 s[NQ][4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[t][ks], q[nq][ks], acc, 0, 0, 0);
+      s[nq][t] = acc;
+    }
+  }
+  float m_new[NQ];
+  bool behind = false;
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    if (MASKED) {
+      const int qp = qpos[nq];
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[nq][t][r] = kb + 16 * t + 4 * g + r <= qp ? s[nq][t][r] : -INFINITY;
+    }
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      tile_max = fmaxf(tile_max, fmaxf(fmaxf(s[nq][t][0], s[nq][t][1]), fmaxf(s[nq][t][2], s[nq][t][3])));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    m_new[nq] = fmaxf(m[nq], tile_max * c);
+    behind = behind || m_new[nq] > m[nq] + RESCALE_SLACK;
+  }
+  if (__builtin_amdgcn_ballot_w64(behind) != 0) {
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      float alpha = m_new[nq] == -INFINITY ? 1.f : exp2f(m[nq] - m_new[nq]);
+      m[nq] = m_new[nq];
+      l[nq] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[nq][dt][r] *= alpha;
+    }
+  }
+  bf16x8 pop[NQ][2];
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    const float m_use = m[nq] == -INFINITY ? 0.f : m[nq];
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float p = __builtin_amdgcn_exp2f(fmaf(s[nq][t][r], c, -m_use));
+        psum += p;
+        pop[nq][t >> 1][4 * (t & 1) + r] = (bf16_t)p;
+      }
+    l[nq] += psum;
+  }
+  const bool ragged = MASKED && kb + 64 > valid_end;
+#pragma unroll
+  for (int dt = 0; dt < ND; ++dt) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      bf16x4 v0 = blk.v[dt][2 * half], v1 = blk.v[dt][2 * half + 1];
+      if (ragged) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (kb + 32 * half + 4 * g + r >= valid_end) v0[r] = (bf16_t)0.f;
+          if (kb + 32 * half + 16 + 4 * g + r >= valid_end) v1[r] = (bf16_t)0.f;
+        }
+      }
+      bf16x8 vop = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq)
+        o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[nq][half], o[nq][dt], 0, 0, 0);
+    }
+  }
+}
+
+#if BT_HEAD_DIM == 64
+// The same for heads of 64 without a window, with the keys and values shared through LDS: a
+// block of 64 positions (8 KiB of keys, 8 KiB of values, each one contiguous plane of the cache)
+// is brought in ONCE per work-group, one or two 16-byte pieces per thread, while the block
+// before it is being multiplied; every wave then reads its MFMA operands from LDS.  With each
+// wave loading its own operands from memory the kernel was bound by what one compute unit can
+// pull (about 25 GB/s): the four or eight waves asked for the same bytes four or eight times.
+//   keys:   row r (128 bytes) keeps its 16-byte chunk c at c ^ ((r >> 1) & 7): the 16 lanes of
+//           a ds_read_b128 that read one chunk of 16 consecutive rows then hit different banks;
+//   values: the 512 bytes of a group of four positions are followed by 128 bytes of padding, so
+//           that the groups g and g + 1 a ds_read_b64 touches together lie in different banks.
+#define SHARED_K_BYTES (64 * 128)
+#define SHARED_V_GROUP 640
+#define SHARED_V_BYTES (16 * SHARED_V_GROUP)
+#define SHARED_STAGE (SHARED_K_BYTES + SHARED_V_BYTES)
+
+template <bool PAIRED>
+__global__ void __launch_bounds__((PAIRED ? 2 : 1) * PREFILL_WAVES * 64)
+attention_prefill_shared_kernel(AttnArgs a) {
+  constexpr int THREADS = (PAIRED ? 2 : 1) * PREFILL_WAVES * 64;
+  constexpr int PIECES = 512 / THREADS;   // 16-byte pieces of an 8 KiB plane per thread
+  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][SHARED_STAGE];
+  const int tid = threadIdx.x, lane = tid & 63;
+  int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int i16 = lane & 15, g = lane >> 4;
+  // numbering of work-groups, pairing of tiles: as in attention_prefill_kernel
+  const int group = a.q_heads / a.kv.kv_heads;
+  const int q_tiles = (a.max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES;
+  const int pairs = PAIRED ? (q_tiles + 1) / 2 : q_tiles;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int unit = (slot / (group * pairs)) * 8 + xcd;
+  if (unit >= a.n_seqs * a.kv.kv_heads) return;             // the whole work-group
+  const int within = slot % (group * pairs);
+  const int seq = unit / a.kv.kv_heads, kv_head = unit % a.kv.kv_heads;
+  const int head = kv_head * group + within % group;
+  const int pair = within / group, late = q_tiles - 1 - pair;
+  const int off = a.seq_off[seq], count = a.seq_off[seq + 1] - off, start = a.seq_start[seq];
+  // the blocks the work-group walks: up to the last query of its later tile that exists
+  const int first_tile = PAIRED && pair < late ? pair : late;   // the earlier tile of the two (or the only one)
+  if (first_tile * PREFILL_QUERIES >= count) return;            // the whole work-group: no query of this sequence here
+  const int last_tile = late * PREFILL_QUERIES < count ? late : first_tile;
+  const int reach = (last_tile + 1) * PREFILL_QUERIES < count ? (last_tile + 1) * PREFILL_QUERIES : count;
+  const int n_blocks = (start + reach + BT_KV_BLOCK - 1) / BT_KV_BLOCK;
+  // this wave's queries; a wave without any still moves its share of every block
+  const bool second = PAIRED && wave >= PREFILL_WAVES;
+  const int q_tile = second ? pair : late;
+  wave &= PREFILL_WAVES - 1;
+  const int q0 = q_tile * PREFILL_QUERIES + wave * PREFILL_QUERIES_PER_WAVE;
+  const bool active = !(second && pair == late) && q0 < count;
+  const bf16_t* Q = static_cast<const bf16_t*>(a.q);
+
+  int qpos[PREFILL_NQ], tok[PREFILL_NQ];
+  bf16x8 q[PREFILL_NQ][NKS];
+  floatx4 o[PREFILL_NQ][ND];
+  float m[PREFILL_NQ], l[PREFILL_NQ];
+#pragma unroll
+  for (int nq = 0; nq < PREFILL_NQ; ++nq) {
+    int qi = q0 + nq * 16 + i16;
+    bool exists = active && qi < count;
+    qpos[nq] = exists ? start + qi : -1;
+    tok[nq] = off + (exists ? qi : count - 1);
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      q[nq][ks] = load_bf16x8(Q + (int64_t)tok[nq] * a.ldq + head * HD + ks * 32 + g * 8);
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) o[nq][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    m[nq] = -INFINITY;
+    l[nq] = 0.f;
+  }
+  const int last = q0 + PREFILL_QUERIES_PER_WAVE < count ? q0 + PREFILL_QUERIES_PER_WAVE : count;
+  const int hi = active ? start + last : 0;     // one past the position of this wave's last query
+  const int valid_end = start + count;
+  const float c = a.scale * LOG2_E;
+  const int whole_until = start + q0 + 1;       // tiles ending here or before are seen whole
+  const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
+  const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
+
+  int4v kreg[PIECES], vreg[PIECES];
+  auto fetch = [&](int block_index) {
+    int64_t plane = tile_plane(a, seq, kv_head, block_index * BT_KV_BLOCK);
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) {
+      int piece = tid + u * THREADS;
+      kreg[u] = *reinterpret_cast<const int4v*>(keys + plane + piece * 8);
+      vreg[u] = *reinterpret_cast<const int4v*>(values + plane + piece * 8);
+    }
+  };
+  auto stash = [&](unsigned char* stage) {
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) {
+      int piece = tid + u * THREADS;
+      int row = piece >> 3, chunk = piece & 7;
+      *reinterpret_cast<int4v*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4)) = kreg[u];
+      int grp = piece >> 5, inside = piece & 31;
+      *reinterpret_cast<int4v*>(stage + SHARED_K_BYTES + grp * SHARED_V_GROUP + inside * 16) = vreg[u];
+    }
+  };
+  fetch(0);
+  stash(lds[0]);
+  __syncthreads();
+  for (int j = 0; j < n_blocks; ++j) {
+    const bool more = j + 1 < n_blocks;
+    if (more) fetch(j + 1);
+    const unsigned char* stage = lds[j & 1];
+    const int kb = j * BT_KV_BLOCK;
+    if (kb < hi) {
+      BlockOperands blk;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          int row = 16 * t + i16, chunk = ks * 4 + g;
+          blk.k[t][ks] = *reinterpret_cast<const bf16x8*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
+        }
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt) {
+        const unsigned char* column = stage + SHARED_K_BYTES + (dt * 16 + i16) * 8;
+#pragma unroll
+        for (int quarter = 0; quarter < 4; ++quarter)
+          blk.v[dt][quarter] = *reinterpret_cast<const bf16x4*>(column + (4 * quarter + g) * SHARED_V_GROUP);
+      }
+      if (kb + 64 <= whole_until)
+        attend_block<PREFILL_NQ, false>(blk, kb, valid_end, qpos, c, q, o, m, l);
+      else
+        attend_block<PREFILL_NQ, true>(blk, kb, valid_end, qpos, c, q, o, m, l);
+    }
+    if (more) stash(lds[(j + 1) & 1]);
+    __syncthreads();   // block j + 1 is in place, and everyone is done with block j before it is overwritten
+  }
+  if (!active) return;
+  bf16_t* out = static_cast<bf16_t*>(a.out);
+#pragma unroll
+  for (int nq = 0; nq < PREFILL_NQ; ++nq) {
+    float total = l[nq];
+    total += __shfl_xor(total, 16, 64);
+    total += __shfl_xor(total, 32, 64);
+    float inv = total > 0.f ? 1.0f / total : 0.f;
+    if (qpos[nq] < 0) continue;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+      bf16x4 packed = {(bf16_t)(o[nq][dt][0] * inv), (bf16_t)(o[nq][dt][1] * inv), (bf16_t)(o[nq][dt][2] * inv),
+                       (bf16_t)(o[nq][dt][3] * inv)};
+      *reinterpret_cast<bf16x4*>(out + (int64_t)tok[nq] * a.ldo + head * HD + dt * 16 + 4 * g) = packed;
+    }
+  }
+}
+#endif  // BT_HEAD_DIM == 64
+
 // Eight waves: measured against sixteen and four at batches 1 to 64 (contexts of 500 to 900), eight
 // are never slower, and at batch 64 a compute unit then holds two work-groups, so that one's
 // reduction overlaps the other's loads (57 -> 42 us).
@@ -443,6 +686,15 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
   const int64_t groups = 8 * units_per_xcd * group * (paired ? (q_tiles + 1) / 2 : q_tiles);
   if (groups > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: %lld work-groups are too many", (long long)groups);
   dim3 grid((unsigned)groups);
+#if BT_HEAD_DIM == 64
+  if (args->window == 0) {    // keys and values shared through LDS
+    if (paired)
+      hipLaunchKernelGGL(attention_prefill_shared_kernel<true>, grid, dim3(2 * PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);
+    else
+      hipLaunchKernelGGL(attention_prefill_shared_kernel<false>, grid, dim3(PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);
+    return bt_check_launch("attention_prefill_bf16");
+  }
+#endif
   if constexpr (HD <= 64) {   // (the paired form is not even built for larger heads)
     if (paired) {
       hipLaunchKernelGGL(attention_prefill_kernel<true>, grid, dim3(2 * PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);

@@ -184,6 +184,8 @@ ATTN_CASES = [
     (2, 2, 64, [300, 129], [300, 2], 50),             # window
     (5, 5, 80, [33], [33], 0),
     (2, 1, 128, [260, 31], [1, 1], 100),              # decode with a window
+    (4, 2, 64, [200, 64, 65, 131], [40, 64, 1, 131], 0),   # heads of 64 without a window: keys and values go through LDS
+    (3, 3, 64, [33, 700], [33, 129], 0),
 ]
 
 

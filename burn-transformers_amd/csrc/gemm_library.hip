@@ -5,6 +5,7 @@
 //   EPI_STORE     bfloat16 out = acc + bias                      (bias stays float32)
 //   EPI_ACT       bfloat16 out = gelu_tanh(acc + bias)           (the library's GELU is the tanh form)
 //   EPI_RESIDUAL  float32 out += acc + bias, in place            (C = D = the residual stream, beta = 1)
+//   EPI_F32       float32 out = acc + bias                       (one split only: logits of many rows)
 // Other epilogues (erf GELU, split partial sums, the scatter into the paged cache) are refused
 // here; callers keep the hand-written kernels for them.
 //
@@ -90,7 +91,7 @@ int make_plan(const PlanKey& key, Plan& p) {
     const void* placeholder = &plans;
     BT_LT_CALL("bias", fn_hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &placeholder, sizeof(placeholder)));
   }
-  const hipDataType out_type = mode == EPI_RESIDUAL ? HIP_R_32F : HIP_R_16BF;
+  const hipDataType out_type = (mode == EPI_RESIDUAL || mode == EPI_F32) ? HIP_R_32F : HIP_R_16BF;
   BT_LT_CALL("layout of W", fn_hipblasLtMatrixLayoutCreate(&p.w, HIP_R_16BF, K, N, K));
   BT_LT_CALL("layout of A", fn_hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, K, M, lda));
   BT_LT_CALL("layout of C", fn_hipblasLtMatrixLayoutCreate(&p.c, out_type, N, M, ldo));
@@ -150,7 +151,8 @@ BT_EXPORT int bt_gemm_library_bf16(void* stream, const void* A, int64_t lda, con
   if (handle == nullptr) BT_REFUSE("gemm_library: the library has not been opened");
   if (N <= 0 || K <= 0 || lda < K || epi->ldo < N) BT_REFUSE("gemm_library: sizes M %d N %d K %d do not fit the pitches", M, N, K);
   if (epi->out == nullptr) BT_REFUSE("gemm_library: no output");
-  if (epi->mode != EPI_STORE && epi->mode != EPI_RESIDUAL && !(epi->mode == EPI_ACT && epi->act == ACT_GELU_TANH))
+  if (epi->mode != EPI_STORE && epi->mode != EPI_RESIDUAL && epi->mode != EPI_F32 &&
+      !(epi->mode == EPI_ACT && epi->act == ACT_GELU_TANH))
     BT_REFUSE("gemm_library: epilogue %d (activation %d) is not one the library has", epi->mode, epi->act);
   PlanKey key(M, N, K, lda, epi->ldo, epi->mode, epi->bias != nullptr);
   auto it = plans.find(key);

@@ -155,19 +155,10 @@ class Engine:
             self._meta = torch.empty(max(plan.layout.total * 2, 4096), dtype=torch.int32, device=self.device)
         self._upload(plan.host, self._meta)
         step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
-        if not want_logits:
-            self._forward_without_readout(step)
+        if not want_logits:       # a step whose logits nobody wants still has to fill the cache
+            self.model.forward(step, self.cache, readout=False)
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return self.model.forward(step, self.cache)
-
-    def _forward_without_readout(self, step):
-        """A step whose logits nobody wants still has to fill the cache."""
-        model = self.model
-        from ..parts import Memory
-        stream = model.embedding.embed(step)
-        for entry in model.schedule:
-            memory = Memory(self.cache, entry.cache, entry.writes, step) if entry.cache is not None else None
-            model.blocks[entry.layer].forward(stream, step, memory)
 
     def _run_decode_graph(self, plan):
         key = plan.n_seqs

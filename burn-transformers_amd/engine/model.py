@@ -67,12 +67,15 @@ class CausalLM:
         self.kv_specs = [writers.get(i, (None, None))[0] for i in range(self.cache_entries)]
         self.state_specs = [writers.get(i, (None, None))[1] for i in range(self.cache_entries)]
 
-    def forward(self, step, cache):
-        """Logits (float32 [len(step.sel_rows), vocab]) of the step's wanted rows."""
+    def forward(self, step, cache, readout=True):
+        """Logits (float32 [len(step.sel_rows), vocab]) of the step's wanted rows; with
+        ``readout=False`` the layers only fill the cache and nothing is returned."""
         stream = self.embedding.embed(step)
         for entry in self.schedule:
             memory = Memory(cache, entry.cache, entry.writes, step) if entry.cache is not None else None
             self.blocks[entry.layer].forward(stream, step, memory)
+        if not readout:
+            return None
         hidden = self.final_norm.apply(stream, step, rows=step.sel_rows)
         return self.readout.logits(hidden, step)
 

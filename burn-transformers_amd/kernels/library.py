@@ -161,7 +161,7 @@ def _check_library_products():
 
 
 def _library_takes(epilogue):
-    return epilogue.mode in (EPI_STORE, EPI_RESIDUAL) or (epilogue.mode == EPI_ACT and epilogue.act == 0)
+    return epilogue.mode in (EPI_STORE, EPI_RESIDUAL, EPI_F32) or (epilogue.mode == EPI_ACT and epilogue.act == 0)
 
 
 # --- epilogues -------------------------------------------------------------------------------

@@ -91,6 +91,9 @@ def test_vendor_library_products(m, n, k):
     x = x0.clone().to(DEV)
     K.gemm(a, w, K.epilogue_residual(x, bias), impl="library")
     assert rel_err(x, x0.double() + want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
+    out32 = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    K.gemm(a, w, K.epilogue_f32(out32), impl="library")
+    assert rel_err(out32, want) < 2e-5 * math.sqrt(k)
     with pytest.raises(K.KernelError, match="not one the library has"):
         K.gemm(a, w, K.epilogue_act(out, "gelu_erf", bias), impl="library")
     # what "auto" picks for these rows gives the same

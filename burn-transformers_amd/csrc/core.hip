@@ -526,50 +526,62 @@ __global__ void kv_copy_kernel(T* __restrict__ k_rows, T* __restrict__ v_rows, i
   }
 }
 
-// The same into the cache for bfloat16 rows of a prompt, with wide accesses.  Every token's
-// work-group copies its own key row, eight channels (16 bytes) at a time.  Values lie with four
-// consecutive positions interleaved per channel, so the work-group of the FIRST token of each run
-// of up to four tokens that share such a group (same sequence, consecutive positions, same
-// position / 4) stores the values of the whole run: a full run is one 8-byte store per channel.
+// The same into the cache for bfloat16 rows of a prompt, with wide accesses.  A work-group takes
+// four consecutive tokens of the step.  Keys: every token's row, eight channels (16 bytes) at a
+// time.  Values lie with four consecutive positions interleaved per channel, so they are stored
+// in runs of tokens that share such a group (same sequence, consecutive positions, same
+// position / 4), each by the work-group that holds the run's first token: a full run of four is
+// one 8-byte store per channel, a shorter one (the ends of a prompt that do not fall on a
+// multiple of four) goes element by element.  Four consecutive tokens hold one such first token
+// wherever the prompt starts, so the work-groups have equal work.
 __global__ void __launch_bounds__(256)
 kv_store_bf16_kernel(const bf16_t* __restrict__ k_rows, const bf16_t* __restrict__ v_rows, int64_t ld,
                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, KvView kv, int tokens) {
-  const int t = blockIdx.x;
-  // the neighbours' sequences and positions, all asked for at once (indices clamped into the step)
-  int seqs[5], poss[5];
+  const int t0 = blockIdx.x * 4;
+  // tokens t0 - 1 .. t0 + 6 (indices clamped into the step), all asked for at once
+  int seqs[8], poss[8];
 #pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    int u = t - 1 + i;
+  for (int i = 0; i < 8; ++i) {
+    int u = t0 - 1 + i;
     u = u < 0 ? 0 : (u < tokens ? u : tokens - 1);
     seqs[i] = tok_seq[u];
     poss[i] = tok_pos[u];
   }
-  const int seq = seqs[1], pos = poss[1];
+  const int n = tokens - t0 < 4 ? tokens - t0 : 4;
   const int hd = kv.head_dim, width = kv.kv_heads * hd;
   bf16_t* keys = static_cast<bf16_t*>(kv.keys);
   bf16_t* values = static_cast<bf16_t*>(kv.values);
   typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
-  for (int c = threadIdx.x * 8; c < width; c += 256 * 8) {
+  const int pieces = width >> 3;
+  for (int q = threadIdx.x; q < n * pieces; q += 256) {
+    int i = q / pieces, c = (q - i * pieces) * 8;
     int head = c / hd, channel = c % hd;
+    int seq = seqs[1 + i], pos = poss[1 + i];
     *reinterpret_cast<int4v*>(keys + kv_block_base(kv, seq, pos, head) + key_offset(hd, pos, channel)) =
-        *reinterpret_cast<const int4v*>(k_rows + (int64_t)t * ld + c);
+        *reinterpret_cast<const int4v*>(k_rows + (int64_t)(t0 + i) * ld + c);
   }
-  const bool continues = t > 0 && seqs[0] == seq && poss[0] == pos - 1 && (pos & 3) != 0;
-  if (continues) return;
-  int run = 1;
 #pragma unroll
-  for (int i = 1; i < 4; ++i)
-    if (run == i && t + i < tokens && seqs[1 + i] == seq && poss[1 + i] == pos + i && ((pos + i) & 3) != 0) run = i + 1;
-  for (int c = threadIdx.x; c < width; c += 256) {
-    int head = c / hd, channel = c % hd;
-    int64_t base = kv_block_base(kv, seq, pos, head);     // the run lies in one block
-    if (run == 4) {                                       // then pos is a multiple of four
-      bf16x4 quad = {v_rows[(int64_t)t * ld + c], v_rows[(int64_t)(t + 1) * ld + c],
-                     v_rows[(int64_t)(t + 2) * ld + c], v_rows[(int64_t)(t + 3) * ld + c]};
-      *reinterpret_cast<bf16x4*>(values + base + value_offset(hd, pos, channel)) = quad;
-    } else {
-      for (int i = 0; i < run; ++i)
-        values[base + value_offset(hd, pos + i, channel)] = v_rows[(int64_t)(t + i) * ld + c];
+  for (int i = 0; i < 4; ++i) {
+    if (i >= n) break;
+    const int t = t0 + i, seq = seqs[1 + i], pos = poss[1 + i];
+    const bool continues = t > 0 && seqs[i] == seq && poss[i] == pos - 1 && (pos & 3) != 0;
+    if (continues) continue;     // an earlier token stores this one's values with its own
+    int run = 1;
+#pragma unroll
+    for (int j = 1; j < 4; ++j)
+      if (run == j && t + j < tokens && seqs[1 + i + j] == seq && poss[1 + i + j] == pos + j && ((pos + j) & 3) != 0)
+        run = j + 1;
+    for (int c = threadIdx.x; c < width; c += 256) {
+      int head = c / hd, channel = c % hd;
+      int64_t base = kv_block_base(kv, seq, pos, head);     // the run lies in one block
+      if (run == 4) {                                       // then pos is a multiple of four
+        bf16x4 quad = {v_rows[(int64_t)t * ld + c], v_rows[(int64_t)(t + 1) * ld + c],
+                       v_rows[(int64_t)(t + 2) * ld + c], v_rows[(int64_t)(t + 3) * ld + c]};
+        *reinterpret_cast<bf16x4*>(values + base + value_offset(hd, pos, channel)) = quad;
+      } else {
+        for (int j = 0; j < run; ++j)
+          values[base + value_offset(hd, pos + j, channel)] = v_rows[(int64_t)(t + j) * ld + c];
+      }
     }
   }
 }
@@ -583,7 +595,7 @@ BT_EXPORT int bt_kv_copy(void* stream, int dtype, void* k_rows, void* v_rows, in
   const bool wide = dtype != 0 && to_cache && tokens > 64 && kv->head_dim % 8 == 0 && ld % 8 == 0 &&
                     ((uintptr_t)k_rows & 15) == 0 && ((uintptr_t)kv->keys & 15) == 0 && ((uintptr_t)kv->values & 7) == 0;
   if (wide) {
-    hipLaunchKernelGGL(kv_store_bf16_kernel, grid, block, 0, (hipStream_t)stream, (const bf16_t*)k_rows,
+    hipLaunchKernelGGL(kv_store_bf16_kernel, dim3((tokens + 3) / 4), block, 0, (hipStream_t)stream, (const bf16_t*)k_rows,
                        (const bf16_t*)v_rows, ld, tok_seq, tok_pos, *kv, tokens);
     return bt_check_launch("kv_copy");
   }

@@ -609,7 +609,7 @@ BT_EXPORT int bt_kv_copy(void* stream, int dtype, void* k_rows, void* v_rows, in
 }
 
 // ---------------------------------------------------------------------------------------------
-// Sampling.  One work-group per row of 32-bit logits [rows][vocab].
+// Sampling of each row of 32-bit logits [rows][vocab].
 //   greedy: lowest index of the maximum; log-probability = log_softmax(z)[id]
 //   sample: p = softmax(z / T); id = #{k : c_k < u * c_last} with c the running sum of p in
 //           index order, u = ((mix(seed + gamma * (index + 1)) >> 41) + 0.5) / 2^23,
@@ -623,29 +623,48 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t seed, uint64_t index) {
   return v ^ (v >> 31);
 }
 
-#define SAMPLE_THREADS 1024
+// Two kernels, because one compute unit pulls a row of 50,257 logits (200 KB) no faster than in
+// about 8 us, and the selection needs the row twice over: several work-groups per row (16, or
+// more for vocabularies beyond 65,536) read their part of it ONCE into registers and leave
+// (maximum, its lowest index, sum of exp(z - that maximum)); one work-group per row combines
+// these and, when sampling, walks the one chunk that holds the drawn point.
+#define SAMPLE_THREADS 512
+#define SAMPLE_PER_THREAD 8      // a chunk holds at most SAMPLE_THREADS * SAMPLE_PER_THREAD logits
+#define SAMPLE_CHUNK_MOST (SAMPLE_THREADS * SAMPLE_PER_THREAD)
+
+static int sample_chunks(int vocab) {
+  int needed = (vocab + SAMPLE_CHUNK_MOST - 1) / SAMPLE_CHUNK_MOST;
+  return needed > 16 ? needed : 16;
+}
+
+struct SamplePartial {
+  float top;      // maximum of z / divisor over the chunk
+  float sum;      // sum of exp(z / divisor - top)
+  int arg;        // lowest index of the maximum
+  int pad;
+};
 
 __global__ void __launch_bounds__(SAMPLE_THREADS)
-sample_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int sample, float temperature,
-              uint64_t seed, uint64_t first_draw, const int* __restrict__ draw_rows,
-              int* __restrict__ ids, float* __restrict__ logp) {
+sample_chunks_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int chunk_len, float divisor,
+                     SamplePartial* __restrict__ partials) {
   __shared__ float scratch[32];
-  __shared__ float seg_sum[SAMPLE_THREADS];
   __shared__ int best_index[SAMPLE_THREADS / 64];
   __shared__ float best_value[SAMPLE_THREADS / 64];
-  __shared__ int chosen;
-  int row = blockIdx.x, tid = threadIdx.x;
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
   const float* z = logits + (int64_t)row * ld;
-  // the logits are divided by the temperature only when sampling
-  float divisor = sample ? temperature : 1.0f;
-
+  const int lo = chunk * chunk_len, hi = lo + chunk_len < vocab ? lo + chunk_len : vocab;
+  float v[SAMPLE_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < SAMPLE_PER_THREAD; ++i) {
+    int k = lo + tid + i * SAMPLE_THREADS;
+    v[i] = k < hi ? z[k] / divisor : -INFINITY;
+  }
   // maximum and its lowest index; a thread sees its indices in rising order, so `>` keeps the lowest
   float top = -INFINITY;
   int arg = 0x7fffffff;
-  for (int k = tid; k < vocab; k += SAMPLE_THREADS) {
-    float v = z[k] / divisor;
-    if (v > top) { top = v; arg = k; }
-  }
+#pragma unroll
+  for (int i = 0; i < SAMPLE_PER_THREAD; ++i)
+    if (v[i] > top) { top = v[i]; arg = lo + tid + i * SAMPLE_THREADS; }
   for (int o = 32; o > 0; o >>= 1) {
     float ov = __shfl_xor(top, o, 64);
     int oa = __shfl_xor(arg, o, 64);
@@ -654,63 +673,108 @@ sample_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int sampl
   if ((tid & 63) == 0) { best_value[tid >> 6] = top; best_index[tid >> 6] = arg; }
   __syncthreads();
   top = best_value[0]; arg = best_index[0];
-  for (int w = 1; w < SAMPLE_THREADS / 64; ++w) {
+  for (int w = 1; w < SAMPLE_THREADS / 64; ++w)
     if (best_value[w] > top || (best_value[w] == top && best_index[w] < arg)) { top = best_value[w]; arg = best_index[w]; }
+  float mine = 0.f;
+  if (top != -INFINITY) {
+#pragma unroll
+    for (int i = 0; i < SAMPLE_PER_THREAD; ++i) mine += expf(v[i] - top);   // exp(-inf) = 0 beyond the chunk
   }
+  float total = block_sum(mine, scratch);
+  if (tid == 0) partials[row * gridDim.x + chunk] = SamplePartial{top, total, arg, 0};
+}
 
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_select_kernel(const float* __restrict__ logits, int64_t ld, int vocab, int chunk_len, int chunks, int sample,
+                     float divisor, uint64_t seed, uint64_t first_draw, const int* __restrict__ draw_rows,
+                     const SamplePartial* __restrict__ partials, int* __restrict__ ids, float* __restrict__ logp) {
+  __shared__ float seg_sum[SAMPLE_THREADS];
+  __shared__ int scratch_count[32];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* z = logits + (int64_t)row * ld;
+  const SamplePartial* part = partials + row * chunks;
+  // every thread combines the few partial results itself: no exchange needed
+  float top = -INFINITY;
+  int arg = 0x7fffffff;
+  for (int c = 0; c < chunks; ++c)
+    if (part[c].top > top) { top = part[c].top; arg = part[c].arg; }   // chunks in index order: `>` keeps the lowest
+  auto scaled = [&](int c) { return part[c].top == -INFINITY ? 0.f : part[c].sum * expf(part[c].top - top); };
+  float total = 0.f;
+  for (int c = 0; c < chunks; ++c) total += scaled(c);                  // in index order
   if (!sample) {
-    float mine = 0.f;
-    for (int k = tid; k < vocab; k += SAMPLE_THREADS) mine += expf(z[k] - top);
-    float total = block_sum(mine, scratch);
     if (tid == 0) {
       ids[row] = arg;
       logp[row] = z[arg] - top - logf(total);
     }
     return;
   }
-
-  // each thread owns one contiguous segment of the vocabulary, so that prefix sums run in index order
-  int seg = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  int lo = tid * seg, hi = lo + seg < vocab ? lo + seg : vocab;
-  float mine = 0.f;
-  for (int k = lo; k < hi; ++k) mine += expf(z[k] / divisor - top);
-  seg_sum[tid] = mine;
-  float total = block_sum(mine, scratch);  // also orders the seg_sum writes before the reads below
-  if (tid == 0) {
-    float u = (float)(((double)(splitmix64(seed, first_draw + (uint64_t)(draw_rows ? draw_rows[row] : row)) >> 41) + 0.5) / 8388608.0);
-    float running = 0.f;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) running += seg_sum[t];   // realised total in index order
-    float threshold = u * running;
-    float before = 0.f;
-    int owner = SAMPLE_THREADS - 1;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) {
-      if (before + seg_sum[t] >= threshold) { owner = t; break; }
-      before += seg_sum[t];
-    }
-    int olo = owner * seg, ohi = olo + seg < vocab ? olo + seg : vocab;
-    int k = olo;
-    float c = before;
-    for (; k < ohi; ++k) {
-      c += expf(z[k] / divisor - top);
-      if (!(c < threshold)) break;
-    }
-    if (k >= vocab) k = vocab - 1;
-    chosen = k;
+  const float u = (float)(((double)(splitmix64(seed, first_draw + (uint64_t)(draw_rows ? draw_rows[row] : row)) >> 41) + 0.5) / 8388608.0);
+  const float threshold = u * total;
+  // the chunk in which the running sum reaches the threshold, and the sum before it
+  float before = 0.f;
+  int owner = chunks - 1;
+  for (int c = 0; c < chunks - 1; ++c) {
+    float with = before + scaled(c);
+    if (with >= threshold) { owner = c; break; }
+    before = with;
   }
+  // within it every thread owns a contiguous segment, so that the prefix sums run in index order;
+  // the answer is the number of logits whose running sum stays below the threshold
+  const int lo = owner * chunk_len, hi = lo + chunk_len < vocab ? lo + chunk_len : vocab;
+  const int seg = (hi - lo + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int slo = lo + tid * seg, shi = slo + seg < hi ? slo + seg : hi;
+  float e[SAMPLE_PER_THREAD];
+  float mine = 0.f;
+#pragma unroll
+  for (int i = 0; i < SAMPLE_PER_THREAD; ++i) {
+    e[i] = slo + i < shi ? expf(z[slo + i] / divisor - top) : 0.f;
+    mine += e[i];
+  }
+  seg_sum[tid] = mine;
+  __syncthreads();
+  float c = before;
+  for (int t = 0; t < tid; ++t) c += seg_sum[t];
+  int below = 0;
+#pragma unroll
+  for (int i = 0; i < SAMPLE_PER_THREAD; ++i) {
+    c += e[i];
+    if (slo + i < shi && c < threshold) ++below;
+  }
+  // (running sums rise with the index, so the logits below the threshold are a prefix of the chunk)
+  int count = below;
+  for (int o = 32; o > 0; o >>= 1) count += __shfl_xor(count, o, 64);
+  if ((tid & 63) == 0) scratch_count[tid >> 6] = count;
   __syncthreads();
   if (tid == 0) {
-    ids[row] = chosen;
-    logp[row] = z[chosen] / divisor - top - logf(total);
+    int all = 0;
+    for (int w = 0; w < SAMPLE_THREADS / 64; ++w) all += scratch_count[w];
+    int k = lo + all;
+    if (k >= vocab) k = vocab - 1;
+    ids[row] = k;
+    logp[row] = z[k] / divisor - top - logf(total);
   }
+}
+
+// workspace: device memory for the partial results of every (row, chunk)
+BT_EXPORT int64_t bt_sample_workspace_bytes(int rows, int vocab) {
+  return (int64_t)rows * sample_chunks(vocab > 0 ? vocab : 1) * sizeof(SamplePartial);
 }
 
 BT_EXPORT int bt_sample(void* stream, const float* logits, int64_t ld, int rows, int vocab, int sample,
                         float temperature, uint64_t seed, uint64_t first_draw, const int* draw_rows,
-                        int* ids, float* logp) {
+                        int* ids, float* logp, void* workspace) {
   if (rows <= 0) return BT_OK;
   if (vocab <= 0) BT_REFUSE("sample: vocabulary %d must be positive", vocab);
   if (sample && !(temperature > 0.f)) BT_REFUSE("sample: temperature %g must be positive", (double)temperature);
-  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, logits, ld,
-                     vocab, sample, temperature, seed, first_draw, draw_rows, ids, logp);
+  if (workspace == nullptr) BT_REFUSE("sample: no workspace");
+  const int chunks = sample_chunks(vocab);
+  const int chunk_len = (vocab + chunks - 1) / chunks;
+  // the logits are divided by the temperature only when sampling
+  const float divisor = sample ? temperature : 1.0f;
+  SamplePartial* partials = static_cast<SamplePartial*>(workspace);
+  hipLaunchKernelGGL(sample_chunks_kernel, dim3(chunks, rows), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream,
+                     logits, ld, vocab, chunk_len, divisor, partials);
+  hipLaunchKernelGGL(sample_select_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, logits, ld,
+                     vocab, chunk_len, chunks, sample, divisor, seed, first_draw, draw_rows, partials, ids, logp);
   return bt_check_launch("sample");
 }

@@ -304,14 +304,23 @@ def kv_copy(k_rows, v_rows, tok_seq, tok_pos, kv_view, to_cache):
                                _c_int(1 if to_cache else 0)))
 
 
+_sample_workspaces = {}
+
+
 def sample(logits, ids, logp, temperature=None, seed=0, first_draw=0, draw_rows=None):
     """Greedy (temperature None) or temperature sampling of each row of float32 logits.  Row r uses
     draw number first_draw + (draw_rows[r] if draw_rows is given else r) of the seed's stream."""
     lib = _module("core")
     rows, vocab = logits.shape
     sampling = temperature is not None
+    lib.bt_sample_workspace_bytes.restype = ctypes.c_int64
+    need = lib.bt_sample_workspace_bytes(_c_int(rows), _c_int(vocab))
+    workspace = _sample_workspaces.get(logits.device)
+    if workspace is None or workspace.numel() < need:       # partial results of the first kernel
+        workspace = torch.empty(max(need, 1 << 16), dtype=torch.uint8, device=logits.device)
+        _sample_workspaces[logits.device] = workspace
     _check(lib, lib.bt_sample(_c_ptr(_stream()), _c_ptr(logits.data_ptr()), _c_i64(logits.stride(0)),
                               _c_int(rows), _c_int(vocab), _c_int(1 if sampling else 0),
                               _c_float(temperature if sampling else 1.0), _c_u64(seed & (2 ** 64 - 1)),
                               _c_u64(first_draw & (2 ** 64 - 1)), _c_ptr(_ptr(draw_rows)), _c_ptr(ids.data_ptr()),
-                              _c_ptr(logp.data_ptr())))
+                              _c_ptr(logp.data_ptr()), _c_ptr(workspace.data_ptr())))

@@ -396,12 +396,24 @@ def test_greedy_takes_the_lowest_index_of_the_maximum():
     ref = torch.log_softmax(logits.double(), -1)
     for r in range(4):
         assert abs(float(logp[r]) - float(ref[r, want[r]])) < 1e-4
+    # other widths: a handful of logits, and more than 65,536 (more chunks per row); rows with a pitch
+    for vocab in (3, 100, 70001):
+        wide = torch.randn(5, vocab + 3, generator=gen)
+        wide[1, vocab - 1] = wide[1, 0] = 20.0
+        view = wide.to(DEV)[:, :vocab]
+        ids = torch.empty(5, dtype=torch.int32, device=DEV)
+        logp = torch.empty(5, dtype=torch.float32, device=DEV)
+        K.sample(view, ids, logp)
+        assert ids.tolist() == [int(x) for x in wide[:, :vocab].argmax(-1)] and int(ids[1]) == 0
+        ref = torch.log_softmax(wide[:, :vocab].double(), -1)
+        assert all(abs(float(logp[r]) - float(ref[r, int(ids[r])])) < 1e-4 for r in range(5))
 
 
-def test_sampling_is_the_inverse_cdf_of_the_tempered_softmax():
+@pytest.mark.parametrize("rows,vocab", [(64, 517), (5, 17), (9, 50257), (3, 70001)])
+def test_sampling_is_the_inverse_cdf_of_the_tempered_softmax(rows, vocab):
     import plain_gpt2 as plain
     gen = torch.Generator().manual_seed(1)
-    rows, vocab, temperature, seed, first = 64, 517, 0.8, 1234567, 40
+    temperature, seed, first = 0.8, 1234567, 40
     logits = torch.randn(rows, vocab, generator=gen) * 3
     ids = torch.empty(rows, dtype=torch.int32, device=DEV)
     logp = torch.empty(rows, dtype=torch.float32, device=DEV)

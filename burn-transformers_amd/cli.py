@@ -42,13 +42,23 @@ def main(argv=None):
     parser.add_argument("max_new_tokens", nargs="?", type=int, default=32)
     parser.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     parser.add_argument("--strategy", choices=["greedy", "sample"], default=None,
-                        help="default: greedy, or sample when --temperature is given")
+                        help="default: greedy, or sample when --temperature, --top-k, --top-p or --min-p is given")
     parser.add_argument("--temperature", type=float, default=None)
     parser.add_argument("--seed", type=int, default=0, help="seed of the sampling stream")
     parser.add_argument("--min-new-tokens", type=int, default=0)
     parser.add_argument("--eos-token-ids", type=lambda s: [int(t) for t in s.split(",") if t], default=[])
     parser.add_argument("--stop-sequences", type=lambda s: [[int(t) for t in q.split(",") if t] for q in s.split(";")],
                         default=[], help="token-id sequences, e.g. 13,198;50256")
+    parser.add_argument("--top-k", type=int, default=None, help="sampling: keep scores >= the k-th greatest")
+    parser.add_argument("--top-p", type=float, default=None, help="sampling: nucleus mass in (0, 1]")
+    parser.add_argument("--min-p", type=float, default=None, help="sampling: keep p >= min_p * max p")
+    parser.add_argument("--repetition-penalty", type=float, default=1.0)
+    parser.add_argument("--presence-penalty", type=float, default=0.0)
+    parser.add_argument("--frequency-penalty", type=float, default=0.0)
+    parser.add_argument("--additive-penalty-scope", choices=["generated", "prompt_and_generated"], default="generated")
+    parser.add_argument("--no-repeat-ngram-size", type=int, default=0)
+    parser.add_argument("--logit-bias", default={}, help="token:bias pairs, e.g. 50256:-100,13:1.5",
+                        type=lambda s: {int(k): float(v) for k, v in (pair.split(":") for pair in s.split(",") if pair)})
     parser.add_argument("--prefill-chunk-size", type=int, default=None)
     parser.add_argument("--batch-size", type=int, default=None, help="most prompts that start together")
     parser.add_argument("--max-tokens", type=int, default=None, help="cache size in tokens (default: what the prompts need)")
@@ -66,11 +76,15 @@ def main(argv=None):
         with open(args.random_weights) as handle:
             bt.write_random_model(args.model_dir, json.load(handle), args.weights_seed)
     prompts, tokenizer = parse_prompts(args.prompt, args.model_dir)
-    strategy = args.strategy or ("sample" if args.temperature is not None else "greedy")
+    wants_sampling = any(v is not None for v in (args.temperature, args.top_k, args.top_p, args.min_p))
+    strategy = args.strategy or ("sample" if wants_sampling else "greedy")
     config = bt.GenerationConfig(
         max_new_tokens=args.max_new_tokens, min_new_tokens=args.min_new_tokens, strategy=strategy,
         temperature=args.temperature if args.temperature is not None else 1.0, seed=args.seed,
-        eos_token_ids=args.eos_token_ids, stop_sequences=args.stop_sequences)
+        eos_token_ids=args.eos_token_ids, stop_sequences=args.stop_sequences, top_k=args.top_k, top_p=args.top_p,
+        min_p=args.min_p, repetition_penalty=args.repetition_penalty, presence_penalty=args.presence_penalty,
+        frequency_penalty=args.frequency_penalty, additive_penalty_scope=args.additive_penalty_scope,
+        no_repeat_ngram_size=args.no_repeat_ngram_size, logit_bias=args.logit_bias)
     model = bt.load_model(args.model_dir, dtype=args.dtype)
     need = sum((len(p) + args.max_new_tokens + 63) // 64 * 64 for p in prompts)
     engine = bt.Engine(model, max_tokens=args.max_tokens or need)

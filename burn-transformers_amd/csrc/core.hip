@@ -8,6 +8,8 @@
 // everything that is not an MFMA kernel, and the tests use the matrix product and the
 // attention here as the slow twins of the MFMA kernels.
 
+#include <float.h>
+
 #include "host.h"
 #include "epilogue.h"
 #include "attention.h"
@@ -777,4 +779,291 @@ BT_EXPORT int bt_sample(void* stream, const float* logits, int64_t ld, int rows,
   hipLaunchKernelGGL(sample_select_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream, logits, ld,
                      vocab, chunk_len, chunks, sample, divisor, seed, first_draw, draw_rows, partials, ids, logp);
   return bt_check_launch("sample");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Selection with processing of the logits (src/generation.rs:18-44), for requests that ask for more
+// than plain greedy or temperature sampling.  One work-group of 1,024 threads holds a whole row in
+// registers (thread t owns the indices t, t + 1024, ...), so the row is read once however many
+// steps follow:
+//   1. z += bias                                          (dense vector, zeros where none is set)
+//   2. repetition: seen anywhere ? (z < 0 ? z r : z / r)  then  z -= clamp(f c) + p [c > 0]
+//   3. sampling only: z /= T;   4. z = min(z, FLT_MAX) where 1-3 can overflow
+//   5. banned tokens (n-gram followers, end-of-sequence before min_new_tokens) become -inf
+//   6. sampling only: top-k (scores >= the k-th greatest; ties survive), top-p (ranked by score,
+//      an item survives when the mass before it is below p; items tied with the last survivor
+//      survive too), min-p (p_i >= min_p max p)
+//   7. greedy: lowest index of the maximum; sampling: #{k : c_k < u c_last}, c the running sum of
+//      the surviving exp(z - max) in index order; log-probability under the processed distribution
+// Thresholds are found by bisection on the bits of the scores (32 counting passes over registers);
+// nothing is sorted.
+// ---------------------------------------------------------------------------------------------
+struct ProcessArgs {
+  const float* logits;
+  int64_t ld;
+  int vocab;
+  const float* bias;          // [vocab] or null
+  const int* counts_all;      // [batch rows][vocab]: occurrences in prompt and output, or null
+  const int* counts_add;      // [batch rows][vocab]: what the additive penalties count, or null
+  int64_t counts_ld;
+  const int* batch_rows;      // [rows]: number of the row in the batch as it started; null = the row itself
+  const int* ban_ids;         // banned tokens of row r: ban_ids[ban_offsets[r] .. ban_offsets[r + 1]); null = none
+  const int* ban_offsets;
+  float repetition, presence, frequency;
+  int sample;
+  float temperature;
+  int clamp;
+  int top_k;                  // 0 = off
+  float top_p;                // >= 1 = off
+  float min_p;                // <= 0 = off
+  uint64_t seed, first_draw;
+  int* ids;
+  float* logp;
+};
+
+#define SELECT_THREADS 1024
+#define SELECT_WAVES (SELECT_THREADS / 64)
+
+__device__ __forceinline__ unsigned int ordered_key(float f) {   // larger float <=> larger key
+  unsigned int b = __float_as_uint(f);
+  return b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+
+template <int PER>
+__global__ void __launch_bounds__(SELECT_THREADS)
+select_processed_kernel(ProcessArgs a) {
+  __shared__ unsigned int ban_bits[2048];                 // one bit per token up to 65,536
+  __shared__ float wave_f[SELECT_WAVES];
+  __shared__ int wave_i[SELECT_WAVES];
+  __shared__ float round_part[SELECT_WAVES][PER];
+  __shared__ float round_sum[PER];
+  __shared__ float shared_f[2];
+  __shared__ int shared_i[2];
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int brow = a.batch_rows ? a.batch_rows[row] : row;
+  const int vocab = a.vocab;
+
+  auto block_sum_f = [&](float v) {
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) wave_f[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < SELECT_WAVES; ++w) total += wave_f[w];
+    return total;
+  };
+  auto block_sum_i = [&](int v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    __syncthreads();
+    if (lane == 0) wave_i[wave] = v;
+    __syncthreads();
+    int total = 0;
+    for (int w = 0; w < SELECT_WAVES; ++w) total += wave_i[w];
+    return total;
+  };
+  auto block_max_f = [&](float v) {
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) wave_f[wave] = v;
+    __syncthreads();
+    float top = wave_f[0];
+    for (int w = 1; w < SELECT_WAVES; ++w) top = fmaxf(top, wave_f[w]);
+    return top;
+  };
+
+  for (int i = tid; i < 2048; i += SELECT_THREADS) ban_bits[i] = 0u;
+  __syncthreads();
+  if (a.ban_ids != nullptr)
+    for (int j = a.ban_offsets[row] + tid; j < a.ban_offsets[row + 1]; j += SELECT_THREADS)
+      atomicOr(&ban_bits[a.ban_ids[j] >> 5], 1u << (a.ban_ids[j] & 31));
+  __syncthreads();
+
+  // steps 1 to 5; slots beyond the vocabulary hold -inf like banned tokens
+  const float* zrow = a.logits + (int64_t)row * a.ld;
+  float z[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int k = tid + i * SELECT_THREADS;
+    float v = -INFINITY;
+    if (k < vocab) {
+      v = zrow[k];
+      if (a.bias != nullptr) v += a.bias[k];
+      if (a.counts_all != nullptr && a.repetition != 1.0f && a.counts_all[(int64_t)brow * a.counts_ld + k] > 0)
+        v = v < 0.f ? v * a.repetition : v / a.repetition;
+      if (a.counts_add != nullptr) {
+        const int c = a.counts_add[(int64_t)brow * a.counts_ld + k];
+        if (a.frequency != 0.f) v -= fminf(fmaxf(a.frequency * (float)c, -FLT_MAX), FLT_MAX);
+        if (a.presence != 0.f && c > 0) v -= a.presence;
+      }
+      if (a.sample) v /= a.temperature;
+      if (a.clamp) v = fminf(v, FLT_MAX);
+      if (ban_bits[k >> 5] & (1u << (k & 31))) v = -INFINITY;
+    }
+    z[i] = v;
+  }
+
+  // the maximum and its lowest index
+  float top = -INFINITY;
+  int arg = 0x7fffffff;
+#pragma unroll
+  for (int i = 0; i < PER; ++i)
+    if (z[i] > top) { top = z[i]; arg = tid + i * SELECT_THREADS; }   // rising indices: `>` keeps the lowest
+  for (int o = 32; o > 0; o >>= 1) {
+    float ov = __shfl_xor(top, o, 64);
+    int oa = __shfl_xor(arg, o, 64);
+    if (ov > top || (ov == top && oa < arg)) { top = ov; arg = oa; }
+  }
+  __syncthreads();
+  if (lane == 0) { wave_f[wave] = top; wave_i[wave] = arg; }
+  __syncthreads();
+  top = wave_f[0]; arg = wave_i[0];
+  for (int w = 1; w < SELECT_WAVES; ++w)
+    if (wave_f[w] > top || (wave_f[w] == top && wave_i[w] < arg)) { top = wave_f[w]; arg = wave_i[w]; }
+  if (top == -INFINITY) {            // every token is excluded: nothing can be chosen
+    if (tid == 0) { a.ids[row] = 0; a.logp[row] = -INFINITY; }
+    return;
+  }
+
+  // step 6a: the k-th greatest score, bit by bit: the largest T that at least k scores reach
+  if (a.sample && a.top_k > 0 && a.top_k < vocab) {
+    unsigned int threshold = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned int candidate = threshold | (1u << bit);
+      int mine = 0;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) mine += ordered_key(z[i]) >= candidate ? 1 : 0;
+      if (block_sum_i(mine) >= a.top_k) threshold = candidate;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (ordered_key(z[i]) < threshold) z[i] = -INFINITY;
+  }
+
+  // from here on a slot holds e = exp(z - max): 1 for the maximum, 0 for what is excluded.  The
+  // order of e is the order of z (scores that round to one e count as tied and survive together),
+  // and min-p is simply e >= min_p.
+#pragma unroll
+  for (int i = 0; i < PER; ++i) z[i] = expf(z[i] - top);
+  if (a.sample && a.top_p < 1.0f) {
+    float mine = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) mine += z[i];
+    const float target = a.top_p * block_sum_f(mine);
+    // the smallest T whose mass strictly above it is below the target; the item at T survives
+    unsigned int threshold = 0xFFFFFFFFu;
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned int candidate = threshold & ~(1u << bit);
+      float above = 0.f;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) above += __float_as_uint(z[i]) > candidate ? z[i] : 0.f;   // e >= 0: its bits order it
+      if (block_sum_f(above) < target) threshold = candidate;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (__float_as_uint(z[i]) < threshold) z[i] = 0.f;
+  }
+  if (a.sample && a.min_p > 0.f) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (z[i] < a.min_p) z[i] = 0.f;
+  }
+
+  // sums of each round of 1,024 consecutive indices, then their total in index order
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    float v = wave_sum(z[i]);
+    if (lane == 0) round_part[wave][i] = v;
+  }
+  __syncthreads();
+  if (tid < PER) {
+    float v = 0.f;
+    for (int w = 0; w < SELECT_WAVES; ++w) v += round_part[w][tid];
+    round_sum[tid] = v;
+  }
+  __syncthreads();
+  float total = 0.f;
+  for (int i = 0; i < PER; ++i) total += round_sum[i];
+
+  if (!a.sample) {
+    if (tid == 0) {
+      a.ids[row] = arg;
+      a.logp[row] = -logf(total);          // the chosen token is the maximum: e = 1
+    }
+    return;
+  }
+  const float u = (float)(((double)(splitmix64(a.seed, a.first_draw + (uint64_t)brow) >> 41) + 0.5) / 8388608.0);
+  const float limit = u * total;
+  // the round in which the running sum reaches the limit, and the sum before it
+  float before = 0.f;
+  int owner = PER - 1;
+  for (int i = 0; i < PER - 1; ++i) {
+    float with = before + round_sum[i];
+    if (with >= limit) { owner = i; break; }
+    before = with;
+  }
+  float mine = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i)
+    if (i == owner) mine = z[i];
+  // running sum over the threads of that round: inside the wave, then over the waves before
+  float scan = mine;
+  for (int o = 1; o < 64; o <<= 1) {
+    float up = __shfl_up(scan, o, 64);
+    if (lane >= o) scan += up;
+  }
+  __syncthreads();
+  if (lane == 63) wave_f[wave] = scan;
+  __syncthreads();
+  float lead = before;
+  for (int w = 0; w < wave; ++w) lead += wave_f[w];
+  const int below = (lead + scan < limit) ? 1 : 0;
+  const int count = block_sum_i(below);
+  int chosen = owner * SELECT_THREADS + count;
+  if (chosen >= vocab) chosen = vocab - 1;
+  // the chosen token's e, from the thread that holds it
+  if (tid == 0) shared_f[0] = 0.f;
+  __syncthreads();
+  if ((chosen & (SELECT_THREADS - 1)) == tid) {
+    float e = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (i == (chosen >> 10)) e = z[i];
+    shared_f[0] = e;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    a.ids[row] = chosen;
+    a.logp[row] = logf(shared_f[0]) - logf(total);
+  }
+  (void)shared_i;
+}
+
+BT_EXPORT int bt_select_processed(void* stream, const ProcessArgs* args, int rows) {
+  if (rows <= 0) return BT_OK;
+  const ProcessArgs& a = *args;
+  if (a.vocab <= 0 || a.vocab > 65536) BT_REFUSE("select_processed: vocabulary %d outside 1..65536 (a row is held in one work-group's registers)", a.vocab);
+  if (a.logits == nullptr || a.ids == nullptr || a.logp == nullptr) BT_REFUSE("select_processed: missing operand");
+  if (a.sample && !(a.temperature > 0.f)) BT_REFUSE("select_processed: temperature %g must be positive", (double)a.temperature);
+  if (!(a.repetition > 0.f)) BT_REFUSE("select_processed: repetition penalty %g must be positive", (double)a.repetition);
+  if ((a.ban_ids == nullptr) != (a.ban_offsets == nullptr)) BT_REFUSE("select_processed: banned tokens need their offsets");
+  if (a.top_k < 0 || !(a.top_p > 0.f) || a.min_p > 1.f) BT_REFUSE("select_processed: top_k %d, top_p %g or min_p %g out of range", a.top_k, (double)a.top_p, (double)a.min_p);
+  hipStream_t s = (hipStream_t)stream;
+  if (a.vocab <= 16 * SELECT_THREADS)
+    hipLaunchKernelGGL(select_processed_kernel<16>, dim3(rows), dim3(SELECT_THREADS), 0, s, a);
+  else
+    hipLaunchKernelGGL(select_processed_kernel<64>, dim3(rows), dim3(SELECT_THREADS), 0, s, a);
+  return bt_check_launch("select_processed");
+}
+
+// counts[rows[i]][ids[i]] += 1 for i < n: the occurrence counts the penalties read
+__global__ void count_tokens_kernel(int* __restrict__ counts, int64_t ld, const int* __restrict__ rows,
+                                    const int* __restrict__ ids, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) atomicAdd(&counts[(int64_t)rows[i] * ld + ids[i]], 1);
+}
+
+BT_EXPORT int bt_count_tokens(void* stream, int* counts, int64_t ld, const int* rows, const int* ids, int n) {
+  if (n <= 0) return BT_OK;
+  hipLaunchKernelGGL(count_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, counts, ld, rows, ids, n);
+  return bt_check_launch("count_tokens");
 }

@@ -63,7 +63,7 @@ def prefill_chunks(prompt_lengths, chunk):
 def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None):
     """Runs one batch that starts together to completion; returns its GeneratedSequences."""
     tracker = GenerationTracker(config, [len(p) for p in prompts])
-    sampler = Sampler(config, len(prompts), engine.device)
+    sampler = Sampler(config, len(prompts), engine.device, engine.model.vocab_size, prompts)
     slots = [engine.open() for _ in prompts]
     open_rows = set(range(len(prompts)))
     try:

@@ -324,3 +324,43 @@ def sample(logits, ids, logp, temperature=None, seed=0, first_draw=0, draw_rows=
                               _c_float(temperature if sampling else 1.0), _c_u64(seed & (2 ** 64 - 1)),
                               _c_u64(first_draw & (2 ** 64 - 1)), _c_ptr(_ptr(draw_rows)), _c_ptr(ids.data_ptr()),
                               _c_ptr(logp.data_ptr()), _c_ptr(workspace.data_ptr())))
+
+
+class ProcessArgs(ctypes.Structure):
+    _fields_ = [("logits", _c_ptr), ("ld", _c_i64), ("vocab", _c_int), ("bias", _c_ptr),
+                ("counts_all", _c_ptr), ("counts_add", _c_ptr), ("counts_ld", _c_i64),
+                ("batch_rows", _c_ptr), ("ban_ids", _c_ptr), ("ban_offsets", _c_ptr),
+                ("repetition", _c_float), ("presence", _c_float), ("frequency", _c_float),
+                ("sample", _c_int), ("temperature", _c_float), ("clamp", _c_int),
+                ("top_k", _c_int), ("top_p", _c_float), ("min_p", _c_float),
+                ("seed", _c_u64), ("first_draw", _c_u64), ("ids", _c_ptr), ("logp", _c_ptr)]
+
+
+def select_processed(logits, ids, logp, *, bias=None, counts_all=None, counts_add=None, batch_rows=None,
+                     ban_ids=None, ban_offsets=None, repetition=1.0, presence=0.0, frequency=0.0,
+                     temperature=None, clamp=False, top_k=0, top_p=1.0, min_p=0.0, seed=0, first_draw=0):
+    """One token per row of float32 logits after bias, penalties, temperature, banned tokens and (when
+    sampling: ``temperature`` given) top-k / top-p / min-p; see ``select_processed_kernel``.
+    ``batch_rows`` (int32) names each row's number in the batch as it started: its row in the
+    count tensors and its draw."""
+    lib = _module("core")
+    rows, vocab = logits.shape
+    counts = counts_all if counts_all is not None else counts_add
+    args = ProcessArgs(
+        logits=logits.data_ptr(), ld=logits.stride(0), vocab=vocab, bias=_ptr(bias),
+        counts_all=_ptr(counts_all), counts_add=_ptr(counts_add), counts_ld=counts.stride(0) if counts is not None else 0,
+        batch_rows=_ptr(batch_rows), ban_ids=_ptr(ban_ids), ban_offsets=_ptr(ban_offsets),
+        repetition=repetition, presence=presence, frequency=frequency,
+        sample=1 if temperature is not None else 0, temperature=temperature if temperature is not None else 1.0,
+        clamp=1 if clamp else 0, top_k=top_k or 0, top_p=top_p if top_p is not None else 1.0,
+        min_p=min_p or 0.0, seed=seed & (2 ** 64 - 1), first_draw=first_draw & (2 ** 64 - 1),
+        ids=ids.data_ptr(), logp=logp.data_ptr())
+    _check(lib, lib.bt_select_processed(_c_ptr(_stream()), ctypes.byref(args), _c_int(rows)))
+
+
+def count_tokens(counts, rows, tokens):
+    """counts[rows[i]][tokens[i]] += 1 (int32 counts on the GPU; rows and tokens: Python lists)."""
+    lib = _module("core")
+    pairs = torch.tensor([list(rows), list(tokens)], dtype=torch.int32).to(counts.device, non_blocking=True)
+    _check(lib, lib.bt_count_tokens(_c_ptr(_stream()), _c_ptr(counts.data_ptr()), _c_i64(counts.stride(0)),
+                                    _c_ptr(pairs[0].data_ptr()), _c_ptr(pairs[1].data_ptr()), _c_int(len(rows))))

@@ -1,6 +1,9 @@
 """Token selection on the GPU: greedy (lowest index of the maximum) or temperature sampling by
 inverse CDF with SplitMix64 uniforms, and the log-probability of the chosen token under the
-distribution that was used (src/generation.rs:655-664, 732-743, 1148-1165).
+distribution that was used (src/generation.rs:655-664, 732-743, 1148-1165).  A configuration
+that asks for more (logit bias, repetition / presence / frequency penalties, banned n-grams,
+end-of-sequence held back until min_new_tokens, top-k, top-p, min-p; src/generation.rs:18-44)
+goes through one kernel that holds a row in registers and applies them in the reference's order.
 
 Draw numbering follows the reference (src/generation.rs:667-699): every selection over a batch
 that started with B rows reserves B draws, finished rows included, so the row that started as
@@ -28,25 +31,66 @@ def interior_unit(bits):
 
 
 class Sampler:
-    def __init__(self, config, batch_rows, device):
+    def __init__(self, config, batch_rows, device, vocabulary_size=None, prompts=None):
+        """``prompts`` (token ids of every row of the batch) are needed when the configuration asks
+        for anything that depends on what a row has held so far (penalties, n-gram bans)."""
         self.config, self.batch_rows, self.device = config, batch_rows, device
         self.selections = 0
         # ids and log-probabilities share one buffer so that they come back in one copy
         self.packed = torch.zeros((2, batch_rows), dtype=torch.int32, device=device)
         self.ids, self.logp = self.packed[0], self.packed[1].view(torch.float32)
         self.host = torch.zeros((2, batch_rows), dtype=torch.int32).pin_memory()
+        self.history = self.bias = None
+        if vocabulary_size is not None and config.processes_logits(vocabulary_size):
+            from .history import TokenHistory
+            self.history = TokenHistory(config, vocabulary_size, prompts if prompts is not None
+                                        else [[] for _ in range(batch_rows)], device)
+            if config.logit_bias:
+                bias = torch.zeros(vocabulary_size, dtype=torch.float32)
+                for token, value in config.logit_bias.items():
+                    bias[token] = value
+                self.bias = bias.to(device)
 
     def select(self, logits, rows):
         """One token for each row of ``logits`` (float32 [len(rows), vocab]); ``rows`` are the rows'
         numbers in the batch as it started.  Returns (ids, log-probabilities) as Python lists; this
         is the step's one readback."""
         count = len(rows)
-        draw_rows = None
-        if self.config.sampling:
-            draw_rows = torch.tensor(rows, dtype=torch.int32).to(self.device, non_blocking=True)
-        K.sample(logits, self.ids[:count], self.logp[:count],
-                 temperature=float(self.config.temperature) if self.config.sampling else None,
-                 seed=self.config.seed, first_draw=self.selections * self.batch_rows, draw_rows=draw_rows)
+        config = self.config
+        first_draw = self.selections * self.batch_rows
+        if self.history is None:
+            draw_rows = None
+            if config.sampling:
+                draw_rows = torch.tensor(rows, dtype=torch.int32).to(self.device, non_blocking=True)
+            K.sample(logits, self.ids[:count], self.logp[:count],
+                     temperature=float(config.temperature) if config.sampling else None,
+                     seed=config.seed, first_draw=first_draw, draw_rows=draw_rows)
+        else:
+            # one small upload: the rows' numbers, then where each row's banned tokens start, then those
+            banned = [self.history.banned(row) for row in rows]
+            offsets = [0]
+            for tokens in banned:
+                offsets.append(offsets[-1] + len(tokens))
+            flat = list(rows) + offsets + [t for tokens in banned for t in tokens]
+            table = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=True)
+            has_bans = offsets[-1] > 0
+            K.select_processed(
+                logits, self.ids[:count], self.logp[:count], bias=self.bias,
+                counts_all=self.history.counts_all if config.repetition_penalty != 1.0 else None,
+                counts_add=self.history.additive_counts, batch_rows=table[:count],
+                ban_ids=table[2 * count + 1:] if has_bans else None,
+                ban_offsets=table[count:2 * count + 1] if has_bans else None,
+                repetition=float(config.repetition_penalty), presence=float(config.presence_penalty),
+                frequency=float(config.frequency_penalty),
+                temperature=float(config.temperature) if config.sampling else None,
+                clamp=config.adjusts_logits or (config.sampling and config.temperature < 1.0),
+                top_k=config.top_k if config.sampling and config.top_k is not None else 0,
+                top_p=float(config.top_p) if config.sampling and config.top_p is not None else 1.0,
+                min_p=float(config.min_p) if config.sampling and config.min_p is not None else 0.0,
+                seed=config.seed, first_draw=first_draw)
         self.selections += 1
         self.host.copy_(self.packed)                  # synchronous: the kernels above have finished after it
-        return self.host[0, :count].tolist(), self.host[1].view(torch.float32)[:count].tolist()
+        ids = self.host[0, :count].tolist()
+        if self.history is not None:
+            self.history.record(list(rows), ids)
+        return ids, self.host[1].view(torch.float32)[:count].tolist()

@@ -190,3 +190,80 @@ def log_probability(logits, index, temperature=None):
     if temperature is not None:
         z = z / temperature
     return float(torch.log_softmax(z, dim=-1)[index])
+
+
+# --- processing of the logits before a token is chosen (src/generation.rs:18-44) -------------------
+
+F32_MAX = 3.4028234663852886e38
+
+
+def banned_by_ngrams(tokens, size):
+    """Tokens that would complete an n-gram the row already holds: whatever followed the last
+    size - 1 tokens earlier (src/generation/ngram.rs:1-12, 57-100)."""
+    if size <= 0 or len(tokens) < size - 1:
+        return []
+    prefix = list(tokens[len(tokens) - (size - 1):]) if size > 1 else []
+    out = set()
+    for end in range(size - 1, len(tokens)):            # tokens[end] is the last token of an n-gram
+        if list(tokens[end - (size - 1):end]) == prefix:
+            out.add(tokens[end])
+    return sorted(out)
+
+
+def process_logits(z, sampling, temperature=1.0, logit_bias=None, repetition_penalty=1.0, presence_penalty=0.0,
+                   frequency_penalty=0.0, seen_counts=None, additive_counts=None, banned=()):
+    """Bias, penalties, temperature, overflow clamp, hard constraints, in that order
+    (src/generation.rs:608-640; penalties :838-923; bias :767-795; constraints :797-836)."""
+    z = z.to(torch.float64).clone()
+    adjusts = bool(logit_bias) or repetition_penalty != 1.0 or presence_penalty != 0.0 or frequency_penalty != 0.0
+    for token, bias in (logit_bias or {}).items():
+        z[token] += bias
+    if repetition_penalty != 1.0:
+        seen = seen_counts > 0
+        penalized = torch.where(z < 0, z * repetition_penalty, z / repetition_penalty)
+        z = torch.where(seen, penalized, z)
+    if frequency_penalty != 0.0:
+        z = z - (additive_counts.to(torch.float64) * frequency_penalty).clamp(-F32_MAX, F32_MAX)
+    if presence_penalty != 0.0:
+        z = z - (additive_counts > 0).to(torch.float64) * presence_penalty
+    if sampling:
+        z = z / temperature
+    if adjusts or (sampling and temperature < 1.0):
+        z = z.clamp(max=F32_MAX)
+    for token in banned:
+        z[token] = -math.inf
+    return z
+
+
+def filter_top_k(z, k):
+    """Every score below the k-th greatest becomes -inf; ties with it survive (generation.rs:1189-1208)."""
+    boundary = torch.sort(z, descending=True).values[k - 1]
+    return torch.where(z < boundary, torch.full_like(z, -math.inf), z)
+
+
+def filter_top_p(z, p):
+    """Ranked by score, an item survives when the mass before it is below p (generation.rs:1210-1233).
+    Items with equal scores are ranked by index here; the reference leaves that to its backend's sort."""
+    order = torch.sort(z, descending=True, stable=True).indices
+    mass = torch.softmax(z[order], dim=-1)
+    before = torch.cumsum(mass, dim=-1) - mass
+    keep = torch.zeros_like(z, dtype=torch.bool)
+    keep[order[before < p]] = True
+    return torch.where(keep, z, torch.full_like(z, -math.inf))
+
+
+def filter_min_p(z, min_p):
+    """p_i >= min_p * max p, as z_i >= max z + ln(min_p) (generation.rs:1235-1253)."""
+    threshold = z.max() + math.log(min_p)
+    return torch.where(z < threshold, torch.full_like(z, -math.inf), z)
+
+
+def truncate(z, top_k=None, top_p=None, min_p=None):
+    """top-k, then top-p, then min-p, each only when it is not a no-op (generation.rs:926-948)."""
+    if top_k is not None and top_k < z.numel():
+        z = filter_top_k(z, top_k)
+    if top_p is not None and top_p < 1.0:
+        z = filter_top_p(z, top_p)
+    if min_p is not None and min_p > 0.0:
+        z = filter_min_p(z, min_p)
+    return z

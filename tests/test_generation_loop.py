@@ -9,19 +9,91 @@ from burn_transformers_amd.sampling.tracker import (GenerationTracker, required_
 
 
 def test_generation_config_names_the_first_invalid_field():
-    """src/generation.rs:288 ff."""
+    """src/generation.rs:278-405: ranges of every control, checked in float32."""
     bt.GenerationConfig().validate(100)
+    bt.GenerationConfig(strategy="sample", top_k=100, top_p=1.0, min_p=0.0, repetition_penalty=1.3, presence_penalty=-2.0,
+                        frequency_penalty=0.5, no_repeat_ngram_size=3, logit_bias={99: -5.0},
+                        additive_penalty_scope="prompt_and_generated").validate(100)
     cases = [(dict(max_new_tokens=0), "max_new_tokens"), (dict(min_new_tokens=9, max_new_tokens=3), "min_new_tokens"),
              (dict(strategy="beam"), "strategy"), (dict(temperature=0.0), "temperature"),
-             (dict(temperature=float("inf")), "temperature"), (dict(eos_token_ids=[100]), "eos_token_ids"),
-             (dict(pad_token_id=-1), "pad_token_id"), (dict(stop_sequences=[[]]), "stop_sequences"),
-             (dict(stop_sequences=[[1, 200]]), "stop_sequences"), (dict(top_k=5), "top_k"),
-             (dict(repetition_penalty=1.1), "repetition_penalty")]
+             (dict(temperature=float("inf")), "temperature"), (dict(temperature=1e-46), "temperature"),
+             (dict(eos_token_ids=[100]), "special token 100"), (dict(pad_token_id=-1), "special token -1"),
+             (dict(stop_sequences=[[]]), "stop sequences must not be empty"),
+             (dict(stop_sequences=[[1, 200]]), "special token 200"),
+             (dict(top_k=0), "top_k"), (dict(top_k=101), "top_k"), (dict(top_p=0.0), "top_p"), (dict(top_p=1.5), "top_p"),
+             (dict(min_p=-0.1), "min_p"), (dict(min_p=1.1), "min_p"),
+             (dict(repetition_penalty=0.0), "repetition_penalty"), (dict(repetition_penalty=1e39), "repetition_penalty"),
+             (dict(presence_penalty=float("nan")), "presence_penalty"), (dict(frequency_penalty=1e39), "frequency_penalty"),
+             (dict(additive_penalty_scope="prompt"), "additive_penalty_scope"),
+             (dict(no_repeat_ngram_size=-1), "no_repeat_ngram_size"),
+             (dict(logit_bias={100: 1.0}), "logit_bias token 100"), (dict(logit_bias={3: float("inf")}), "logit_bias for token 3"),
+             # the first invalid field in the reference's order is the one that is named
+             (dict(temperature=0.0, top_k=0), "temperature"), (dict(top_k=0, repetition_penalty=0.0), "top_k")]
     for fields, name in cases:
         with pytest.raises(bt.GenerationError, match=name):
             bt.GenerationConfig(**fields).validate(100)
     with pytest.raises(bt.GenerationError, match="vocabulary_size"):
         bt.GenerationConfig().validate(0)
+
+
+def test_which_configurations_process_the_logits():
+    plain = bt.GenerationConfig()
+    assert not plain.processes_logits(100) and not plain.counts_all and not plain.counts_generated
+    assert not bt.GenerationConfig(strategy="sample", temperature=0.5, top_k=100, top_p=1.0, min_p=0.0).processes_logits(100)
+    assert not bt.GenerationConfig(top_k=5, top_p=0.5).processes_logits(100)          # greedy ignores the warpers
+    assert bt.GenerationConfig(strategy="sample", top_k=5).processes_logits(100)
+    assert bt.GenerationConfig(min_new_tokens=2, eos_token_ids=[1]).processes_logits(100)
+    assert not bt.GenerationConfig(min_new_tokens=2).processes_logits(100)
+    rep = bt.GenerationConfig(repetition_penalty=1.2)
+    assert rep.counts_all and not rep.counts_generated and rep.adjusts_logits
+    freq = bt.GenerationConfig(frequency_penalty=0.1)
+    assert freq.counts_generated and not freq.counts_all
+    assert bt.GenerationConfig(presence_penalty=0.1, additive_penalty_scope="prompt_and_generated").counts_all
+
+
+def test_ngram_index_bans_what_followed_the_same_prefix():
+    """src/generation/ngram.rs:1-12: the index against a direct search of the row."""
+    import random
+    import plain_gpt2 as plain
+    from burn_transformers_amd.sampling.history import NgramIndex
+    rng = random.Random(0)
+    for size in (1, 2, 3, 4):
+        index, tokens = NgramIndex(size), []
+        assert index.banned() == plain.banned_by_ngrams(tokens, size)
+        for _ in range(60):
+            token = rng.randrange(4)
+            tokens.append(token)
+            index.push(token)
+            assert index.banned() == plain.banned_by_ngrams(tokens, size), (size, tokens)
+    assert plain.banned_by_ngrams([1, 2, 3, 1, 2], 3) == [3]          # 1 2 -> 3 was seen
+    assert plain.banned_by_ngrams([1, 2, 3, 1, 2], 2) == [3]          # 2 -> 3
+    assert plain.banned_by_ngrams([5, 6, 5], 1) == [5, 6]             # nothing may repeat
+    assert plain.banned_by_ngrams([5], 3) == []                       # too short for a prefix of two
+
+
+def test_plain_truncation_rules():
+    """Pins of the plain filters on cases worked by hand (src/generation.rs:1189-1253)."""
+    import math
+    import torch
+    import plain_gpt2 as plain
+    z = torch.tensor([1.0, 3.0, 2.0, 3.0, 0.0, -1.0], dtype=torch.float64)
+    kept = lambda t: [i for i, v in enumerate(t.tolist()) if v != -math.inf]
+    assert kept(plain.filter_top_k(z, 1)) == [1, 3]                   # ties with the boundary survive
+    assert kept(plain.filter_top_k(z, 3)) == [1, 2, 3]
+    p = torch.softmax(z, -1)
+    # ranked 1, 3, 2, 0, 4, 5: an item survives when the mass before it is below p
+    assert kept(plain.filter_top_p(z, float(p[1]) * 0.5)) == [1]
+    assert kept(plain.filter_top_p(z, float(p[1]) + 1e-9)) == [1, 3]
+    assert kept(plain.filter_top_p(z, float(p[1] + p[3] + p[2]) + 1e-9)) == [0, 1, 2, 3]
+    assert kept(plain.filter_min_p(z, math.exp(-1.0) - 1e-9)) == [1, 2, 3]     # z >= 3 - 1
+    assert kept(plain.filter_min_p(z, math.exp(-1.0) + 1e-9)) == [1, 3]
+    assert kept(plain.truncate(z, top_k=6, top_p=1.0, min_p=0.0)) == [0, 1, 2, 3, 4, 5]
+    # processing order: bias before the repetition penalty, ban last
+    counts = torch.tensor([1, 0, 0, 0, 0, 2])
+    out = plain.process_logits(z, sampling=True, temperature=2.0, logit_bias={0: 1.0}, repetition_penalty=2.0,
+                               presence_penalty=0.5, frequency_penalty=0.25, seen_counts=counts, additive_counts=counts,
+                               banned=[4])
+    assert out.tolist() == [((1.0 + 1.0) / 2.0 - 0.25 - 0.5) / 2.0, 1.5, 1.0, 1.5, -math.inf, (-1.0 * 2.0 - 0.5 - 0.5) / 2.0]
 
 
 def test_end_of_sequence_beats_stop_sequence_beats_length():

@@ -442,20 +442,25 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
 template <int MT, int NT, int U, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
-                   int K, Epilogue epi) {
+                   int K, Epilogue epi, int tile_columns) {
+  // tile_columns: how many of its 16 * NT output columns a work-group really owns (a multiple of
+  // four).  Fewer than all of them is for balance: 300 work-groups of 16 columns leave 44 of 256
+  // compute units with twice the bytes of the others, 400 of 12 columns leave every unit at most
+  // 24 columns.  The lanes of the columns left out repeat the last real one and store nothing.
   __shared__ __attribute__((aligned(16))) float red[WAVES][MT * NT][64][4];
   static_assert(MT * NT <= WAVES, "one wave finishes each block of the work-group's output");
   // the wave's number is the same in all its lanes: saying so keeps every test on it a scalar
   // branch, which costs no wait for loads in flight (a divergent one does)
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int i16 = lane & 15, g = lane >> 4;
-  const int n_base = blockIdx.x * 16 * NT;
+  const int n_base = blockIdx.x * tile_columns;
+  const int n_end = n_base + tile_columns < N ? n_base + tile_columns : N;   // one past this work-group's last column
   const int split = blockIdx.y, splits = gridDim.y;
   const bf16_t* w_row[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     int n = n_base + nt * 16 + i16;
-    w_row[nt] = W + (int64_t)(n < N ? n : N - 1) * K;
+    w_row[nt] = W + (int64_t)(n < n_end ? n : n_end - 1) * K;
   }
   const bf16_t* a_row[MT];
 #pragma unroll
@@ -518,7 +523,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
   const int mine = wave < blocks ? wave : 0;
   const int out_m = (mine / NT) * 16 + i16, out_n0 = n_base + (mine % NT) * 16 + g * 4;
   EpiloguePrefetch pre = {};
-  if (wave < blocks) pre = epilogue_prefetch(epi, M, N, out_m, out_n0, split);
+  if (wave < blocks) pre = epilogue_prefetch(epi, M, n_end, out_m, out_n0, split);
   multiply(c0);
   for (c0 += stride * U; c0 < chunks; c0 += stride * U) {
     issue(c0);
@@ -536,7 +541,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
     for (int w = 0; w < WAVES; ++w)
 #pragma unroll
       for (int r = 0; r < 4; ++r) v[r] += red[w][wave][lane][r];
-    if (out_m < M) epilogue4_prefetched<bf16_t>(epi, N, out_m, out_n0, v, split, pre);
+    if (out_m < M) epilogue4_prefetched<bf16_t>(epi, n_end, out_m, out_n0, v, split, pre);   // nothing beyond n_end
   }
 }
 
@@ -620,16 +625,41 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  // variant 1 (measurements and tests): one column block per work-group also beyond 16 rows
-  if (M <= 16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 8, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
-  else if (M <= 32 && variant == 1)
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 1, 4, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
-  else if (variant == 1)
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 1, 2, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
-  else if (M <= 32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 2, 4, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
-  else
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 2, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi);
+  // Up to 16 rows: 16, 12 or 8 columns per work-group, whichever leaves the busiest compute unit
+  // the least to pull: work-groups land on the units in whole rounds, and a work-group costs its
+  // slice of K times its columns plus a fixed part (about ten chunks of sixteen columns).
+  // variant 1 (measurements and tests): 16 columns, and one column block also beyond 16 rows;
+  // variants 12 and 8 force that many columns.
+  static int compute_units = 0;
+  if (compute_units == 0) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+      compute_units = 256;
+  }
+  if (M <= 16) {
+    int columns = 16;
+    if (variant == 12 || variant == 8) {
+      columns = variant;
+    } else if (variant == 0) {
+      const int64_t per = ((K + 31) / 32 + splits - 1) / splits;
+      int64_t best = -1;
+      for (int c = 16; c >= 8; c -= 4) {
+        int64_t groups = (int64_t)((N + c - 1) / c) * splits;
+        int64_t cost = ((groups + compute_units - 1) / compute_units) * (per * c + 160);
+        if (best < 0 || cost < best) { best = cost; columns = c; }
+      }
+    }
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 8, 8>), dim3((N + columns - 1) / columns, splits), dim3(512), 0, s, a,
+                       lda, w, M, N, K, *epi, columns);
+  } else if (M <= 32 && variant == 1) {
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, 1, 4, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 16);
+  } else if (variant == 1) {
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, 1, 2, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 16);
+  } else if (M <= 32) {
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, 2, 4, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 32);
+  } else {
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 2, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 32);
+  }
   return bt_check_launch("gemm_skinny_bf16");
 }

@@ -106,15 +106,18 @@ def test_vendor_library_products(m, n, k):
 @pytest.mark.parametrize("m,n,k,splits", [(1, 100, 136, 1), (8, 4800, 1600, 2), (16, 1600, 1600, 4),
                                           (7, 333, 6400, 8), (3, 50, 1760, 1), (16, 517, 1608, 3),
                                           (2, 16, 8, 1), (9, 40, 3400, 1)])
-def test_skinny_gemm_at_decode_sizes(m, n, k, splits):
-    """Up to 16 rows, K with a short last chunk, slices of K that do not divide evenly."""
+@pytest.mark.parametrize("columns", [0, 16, 12, 8])
+def test_skinny_gemm_at_decode_sizes(m, n, k, splits, columns):
+    """Up to 16 rows, K with a short last chunk, slices of K that do not divide evenly; 16, 12 or 8
+    output columns per work-group (0: chosen for balance)."""
+    variant = {0: 0, 16: 1, 12: 12, 8: 8}[columns]
     a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=k, lda=k + 24)
     parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
-    K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl="skinny")
+    K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl="skinny", variant=variant)
     assert rel_err(parts.sum(0), want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
     if splits == 1:
         out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
-        K.gemm(a, w, K.epilogue_act(out, "gelu_tanh", bias), impl="skinny")
+        K.gemm(a, w, K.epilogue_act(out, "gelu_tanh", bias), impl="skinny", variant=variant)
         assert rel_err(out, gelu_tanh(want + bias.cpu().double())) < 6e-3
 
 
@@ -165,7 +168,8 @@ def test_fused_projection_scatters_into_the_cache(impl, dtype, counts):
     want = want + bias.cpu().double()
     q = torch.full((case.n_tokens, n_q), float("nan"), dtype=dt, device=DEV)
     before_k, before_v = case.read_back()
-    K.gemm(a, w, K.epilogue_qkv(q, n_q, n_kv, case.view(), case.tok_seq, case.tok_pos, bias), impl=impl)
+    K.gemm(a, w, K.epilogue_qkv(q, n_q, n_kv, case.view(), case.tok_seq, case.tok_pos, bias), impl=impl,
+           variant=12 if impl == "skinny" and case.n_tokens <= 16 else 0)
     after_k, after_v = case.read_back()
     tol = 2e-6 if dtype == "float32" else 6e-3
     assert rel_err(q, want[:, :n_q]) < tol

@@ -625,11 +625,11 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  // Up to 16 rows: 16, 12 or 8 columns per work-group, whichever leaves the busiest compute unit
+  // Up to 16 rows: 8 to 32 columns per work-group in steps of four, whichever leaves the busiest compute unit
   // the least to pull: work-groups land on the units in whole rounds, and a work-group costs its
   // slice of K times its columns plus a fixed part (about ten chunks of sixteen columns).
   // variant 1 (measurements and tests): 16 columns, and one column block also beyond 16 rows;
-  // variants 12 and 8 force that many columns.
+  // variants 8, 12, ... 32 force that many columns.
   static int compute_units = 0;
   if (compute_units == 0) {
     int device = 0;
@@ -639,19 +639,22 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
   }
   if (M <= 16) {
     int columns = 16;
-    if (variant == 12 || variant == 8) {
+    if (variant >= 8 && variant <= 32 && variant % 4 == 0) {
       columns = variant;
     } else if (variant == 0) {
       const int64_t per = ((K + 31) / 32 + splits - 1) / splits;
       int64_t best = -1;
-      for (int c = 16; c >= 8; c -= 4) {
+      for (int c = 32; c >= 8; c -= 4) {
         int64_t groups = (int64_t)((N + c - 1) / c) * splits;
         int64_t cost = ((groups + compute_units - 1) / compute_units) * (per * c + 160);
         if (best < 0 || cost < best) { best = cost; columns = c; }
       }
     }
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 8, 8>), dim3((N + columns - 1) / columns, splits), dim3(512), 0, s, a,
-                       lda, w, M, N, K, *epi, columns);
+    dim3 grid((N + columns - 1) / columns, splits);
+    if (columns <= 16)
+      hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 8, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi, columns);
+    else       // two column blocks, of which the second is partly left out
+      hipLaunchKernelGGL((gemm_skinny_kernel<1, 2, 8, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi, columns);
   } else if (M <= 32 && variant == 1) {
     hipLaunchKernelGGL((gemm_skinny_kernel<2, 1, 4, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 16);
   } else if (variant == 1) {

@@ -106,11 +106,11 @@ def test_vendor_library_products(m, n, k):
 @pytest.mark.parametrize("m,n,k,splits", [(1, 100, 136, 1), (8, 4800, 1600, 2), (16, 1600, 1600, 4),
                                           (7, 333, 6400, 8), (3, 50, 1760, 1), (16, 517, 1608, 3),
                                           (2, 16, 8, 1), (9, 40, 3400, 1)])
-@pytest.mark.parametrize("columns", [0, 16, 12, 8])
+@pytest.mark.parametrize("columns", [0, 16, 12, 8, 20, 28, 32])
 def test_skinny_gemm_at_decode_sizes(m, n, k, splits, columns):
     """Up to 16 rows, K with a short last chunk, slices of K that do not divide evenly; 16, 12 or 8
-    output columns per work-group (0: chosen for balance)."""
-    variant = {0: 0, 16: 1, 12: 12, 8: 8}[columns]
+    to 32 output columns per work-group (0: chosen for balance)."""
+    variant = 1 if columns == 16 else columns
     a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=k, lda=k + 24)
     parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
     K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl="skinny", variant=variant)

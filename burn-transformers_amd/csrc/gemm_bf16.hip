@@ -625,11 +625,9 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  // Up to 16 rows: 8 to 32 columns per work-group in steps of four, whichever leaves the busiest compute unit
-  // the least to pull: work-groups land on the units in whole rounds, and a work-group costs its
-  // slice of K times its columns plus a fixed part (about ten chunks of sixteen columns).
-  // variant 1 (measurements and tests): 16 columns, and one column block also beyond 16 rows;
-  // variants 8, 12, ... 32 force that many columns.
+  // 8 to 32 columns per work-group in steps of four (one or two column blocks of the kernel),
+  // whichever leaves the busiest compute unit the least to pull: work-groups land on the units in
+  // whole rounds.  Variants 8, 12, ... 32 (measurements and tests) force that many.
   static int compute_units = 0;
   if (compute_units == 0) {
     int device = 0;
@@ -637,32 +635,30 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
         hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
       compute_units = 256;
   }
-  if (M <= 16) {
-    int columns = 16;
-    if (variant >= 8 && variant <= 32 && variant % 4 == 0) {
-      columns = variant;
-    } else if (variant == 0) {
-      const int64_t per = ((K + 31) / 32 + splits - 1) / splits;
-      int64_t best = -1;
-      for (int c = 32; c >= 8; c -= 4) {
-        int64_t groups = (int64_t)((N + c - 1) / c) * splits;
-        int64_t cost = ((groups + compute_units - 1) / compute_units) * (per * c + 160);
-        if (best < 0 || cost < best) { best = cost; columns = c; }
-      }
+  // columns per work-group: the cost of a work-group is what it pulls for one chunk of K (its
+  // columns of the weights and the step's rows of the activations) times its chunks, plus a fixed part
+  int columns = M <= 16 ? 16 : 32;
+  if (variant >= 8 && variant <= 32 && variant % 4 == 0) {
+    columns = variant;
+  } else if (variant == 0) {
+    const int64_t per = ((K + 31) / 32 + splits - 1) / splits;
+    int64_t best = -1;
+    for (int c = 32; c >= 8; c -= 4) {
+      int64_t groups = (int64_t)((N + c - 1) / c) * splits;
+      int64_t cost = ((groups + compute_units - 1) / compute_units) * (per * (c + M) + 160);
+      if (best < 0 || cost < best) { best = cost; columns = c; }
     }
-    dim3 grid((N + columns - 1) / columns, splits);
-    if (columns <= 16)
-      hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 8, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi, columns);
-    else       // two column blocks, of which the second is partly left out
-      hipLaunchKernelGGL((gemm_skinny_kernel<1, 2, 8, 8>), grid, dim3(512), 0, s, a, lda, w, M, N, K, *epi, columns);
-  } else if (M <= 32 && variant == 1) {
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 1, 4, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 16);
-  } else if (variant == 1) {
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 1, 2, 8>), dim3((N + 15) / 16, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 16);
-  } else if (M <= 32) {
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 2, 4, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 32);
-  } else {
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 2, 8>), dim3((N + 31) / 32, splits), dim3(512), 0, s, a, lda, w, M, N, K, *epi, 32);
   }
+  dim3 grid((N + columns - 1) / columns, splits), block(512);
+#define LAUNCH_SKINNY(MT, NT, U) \
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, *epi, columns)
+  if (M <= 16) {
+    if (columns <= 16) LAUNCH_SKINNY(1, 1, 8); else LAUNCH_SKINNY(1, 2, 8);
+  } else if (M <= 32) {
+    if (columns <= 16) LAUNCH_SKINNY(2, 1, 4); else LAUNCH_SKINNY(2, 2, 4);
+  } else {
+    if (columns <= 16) LAUNCH_SKINNY(4, 1, 2); else LAUNCH_SKINNY(4, 2, 2);
+  }
+#undef LAUNCH_SKINNY
   return bt_check_launch("gemm_skinny_bf16");
 }

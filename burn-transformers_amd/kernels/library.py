@@ -232,7 +232,7 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
     library where it is usable and has the epilogue, else tile), or one of "plain", "tile",
     "skinny", "library" to force one.  variant picks one of the tile kernel's forms
     (0: the fastest the operands allow, 1: any K, 2: lean, 3: direct to LDS) or, for the skinny
-    kernel beyond 16 rows, one column block per work-group (1) instead of two (0).
+    kernel, the output columns a work-group owns (8, 12, ... 32; 0: chosen for balance).
     """
     m, k = a.shape
     n = w.shape[0]

@@ -110,7 +110,7 @@ def test_vendor_library_products(m, n, k):
 def test_skinny_gemm_at_decode_sizes(m, n, k, splits, columns):
     """Up to 16 rows, K with a short last chunk, slices of K that do not divide evenly; 16, 12 or 8
     to 32 output columns per work-group (0: chosen for balance)."""
-    variant = 1 if columns == 16 else columns
+    variant = columns
     a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=k, lda=k + 24)
     parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
     K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl="skinny", variant=variant)

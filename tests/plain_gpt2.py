@@ -131,9 +131,10 @@ def block(x, w, layer, cfg, taps=None):
     return y + f
 
 
-def forward(ids, w, cfg, dtype=torch.float64, taps=None):
+def forward(ids, w, cfg, dtype=torch.float64, taps=None, rows=None):
     """Logits [S, V] of one whole sequence: embed, blocks, ln_f, tied readout
-    (src/models/gpt2/model.rs:385-420, 500-513)."""
+    (src/models/gpt2/model.rs:385-420, 500-513).  With ``rows``, only those positions are read out:
+    the selection comes after the final norm and before the product (src/models/shared/logits.rs:58-80)."""
     w = {name: t.to(dtype) for name, t in w.items()}
     ids = torch.as_tensor(ids, dtype=torch.long)
     x = embed(ids, torch.arange(ids.numel()), w["wte.weight"], w["wpe.weight"])
@@ -146,6 +147,8 @@ def forward(ids, w, cfg, dtype=torch.float64, taps=None):
     x = layer_norm(x, w["ln_f.weight"], w["ln_f.bias"], cfg["layer_norm_epsilon"])
     if taps is not None:
         taps["final"] = x
+    if rows is not None:
+        x = x[torch.as_tensor(rows, dtype=torch.long)]
     return x @ w["wte.weight"].t()
 
 

@@ -59,6 +59,8 @@ def main(argv=None):
     parser.add_argument("--no-repeat-ngram-size", type=int, default=0)
     parser.add_argument("--logit-bias", default={}, help="token:bias pairs, e.g. 50256:-100,13:1.5",
                         type=lambda s: {int(k): float(v) for k, v in (pair.split(":") for pair in s.split(",") if pair)})
+    parser.add_argument("--total-length", type=int, default=None,
+                        help="a sequence also ends when prompt and output together hold this many tokens")
     parser.add_argument("--prefill-chunk-size", type=int, default=None)
     parser.add_argument("--batch-size", type=int, default=None, help="most prompts that start together")
     parser.add_argument("--max-tokens", type=int, default=None, help="cache size in tokens (default: what the prompts need)")
@@ -86,10 +88,11 @@ def main(argv=None):
         frequency_penalty=args.frequency_penalty, additive_penalty_scope=args.additive_penalty_scope,
         no_repeat_ngram_size=args.no_repeat_ngram_size, logit_bias=args.logit_bias)
     model = bt.load_model(args.model_dir, dtype=args.dtype)
-    need = sum((len(p) + args.max_new_tokens + 63) // 64 * 64 for p in prompts)
+    grows_to = lambda n: n + args.max_new_tokens if args.total_length is None else min(n + args.max_new_tokens, args.total_length)
+    need = sum((grows_to(len(p)) + 63) // 64 * 64 for p in prompts)
     engine = bt.Engine(model, max_tokens=args.max_tokens or need)
     sequences = bt.generate(engine, prompts, config, prefill_chunk=args.prefill_chunk_size,
-                            batch_size=args.batch_size)
+                            batch_size=args.batch_size, total_length=args.total_length)
     for prompt, sequence in zip(prompts, sequences):
         if args.json:
             print(json.dumps({"prompt_length": sequence.prompt_length, "token_ids": sequence.token_ids,

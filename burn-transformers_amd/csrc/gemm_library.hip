@@ -143,6 +143,38 @@ BT_EXPORT int bt_gemm_library_open(const char* path, int* version) {
   return BT_OK;
 }
 
+// Rows a single library call takes: the heuristic finds no algorithm without a workspace for
+// very tall products (32,768 rows were refused), and rows are independent, so taller ones go in
+// runs of this many.
+constexpr int ROWS_PER_CALL = 4096;
+
+namespace {
+
+// The plan for a run of `M` rows, made at first use; nullptr (with the error set) if there is none.
+Plan* plan_for(int M, int N, int K, int64_t lda, const Epilogue* epi) {
+  PlanKey key(M, N, K, lda, epi->ldo, epi->mode, epi->bias != nullptr);
+  auto it = plans.find(key);
+  if (it == plans.end()) {
+    Plan fresh;
+    if (make_plan(key, fresh)) return nullptr;
+    it = plans.emplace(key, fresh).first;
+  }
+  return &it->second;
+}
+
+int run_rows(hipStream_t stream, Plan& p, const char* A, const void* W, const Epilogue* epi, char* out) {
+  if (epi->bias != nullptr) {
+    const void* bias = epi->bias;
+    BT_LT_CALL("bias", fn_hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));
+  }
+  const float alpha = 1.f;
+  BT_LT_CALL("matmul", fn_hipblasLtMatmul(handle, p.desc, &alpha, W, p.w, A, p.a, &p.beta, out, p.c, out, p.c, &p.algo,
+                                          nullptr, 0, stream));
+  return BT_OK;
+}
+
+}  // namespace
+
 // Not safe for concurrent calls (plans are shared and carry the bias pointer of the last call);
 // the engine issues its kernels from one thread.
 BT_EXPORT int bt_gemm_library_bf16(void* stream, const void* A, int64_t lda, const void* W, int M, int N, int K,
@@ -154,21 +186,21 @@ BT_EXPORT int bt_gemm_library_bf16(void* stream, const void* A, int64_t lda, con
   if (epi->mode != EPI_STORE && epi->mode != EPI_RESIDUAL && epi->mode != EPI_F32 &&
       !(epi->mode == EPI_ACT && epi->act == ACT_GELU_TANH))
     BT_REFUSE("gemm_library: epilogue %d (activation %d) is not one the library has", epi->mode, epi->act);
-  PlanKey key(M, N, K, lda, epi->ldo, epi->mode, epi->bias != nullptr);
-  auto it = plans.find(key);
-  if (it == plans.end()) {
-    Plan fresh;
-    int rc = make_plan(key, fresh);
+  // both plans (full runs and the shorter last one) before anything runs, so that a refusal
+  // leaves the output untouched
+  Plan* full = plan_for(M < ROWS_PER_CALL ? M : ROWS_PER_CALL, N, K, lda, epi);
+  if (full == nullptr) return BT_REFUSED;
+  Plan* last = full;
+  if (M > ROWS_PER_CALL && M % ROWS_PER_CALL != 0) {
+    last = plan_for(M % ROWS_PER_CALL, N, K, lda, epi);
+    if (last == nullptr) return BT_REFUSED;      // (entries of a std::map stay where they are: `full` is still good)
+  }
+  const int64_t out_bytes = (epi->mode == EPI_RESIDUAL || epi->mode == EPI_F32) ? 4 : 2;
+  for (int m0 = 0; m0 < M; m0 += ROWS_PER_CALL) {
+    bool whole = M - m0 >= ROWS_PER_CALL;
+    int rc = run_rows((hipStream_t)stream, whole ? *full : *last, (const char*)A + (int64_t)m0 * lda * 2, W, epi,
+                      (char*)epi->out + (int64_t)m0 * epi->ldo * out_bytes);
     if (rc) return rc;
-    it = plans.emplace(key, fresh).first;
   }
-  Plan& p = it->second;
-  if (epi->bias != nullptr) {
-    const void* bias = epi->bias;
-    BT_LT_CALL("bias", fn_hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));
-  }
-  const float alpha = 1.f;
-  BT_LT_CALL("matmul", fn_hipblasLtMatmul(handle, p.desc, &alpha, W, p.w, A, p.a, &p.beta, epi->out, p.c, epi->out, p.c,
-                                          &p.algo, nullptr, 0, (hipStream_t)stream));
   return BT_OK;
 }

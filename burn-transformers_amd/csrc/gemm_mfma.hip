@@ -1,6 +1,7 @@
-// bfloat16 matrix products on the MFMA units of gfx950, C[M,N] = A[M,K] . W[N,K]^T with 32-bit
-// accumulation.  Both operands are K-contiguous, which is what an MFMA lane wants: eight
-// consecutive K values in one 16-byte load.
+// Matrix products on the MFMA units of gfx950, C[M,N] = A[M,K] . W[N,K]^T with 32-bit
+// accumulation, in bfloat16 and in float (the float instructions multiply and add in full
+// 32-bit: no reduced-precision mode exists in them).  Both operands are K-contiguous, which is
+// what an MFMA lane wants: consecutive K values in one 16-byte load.
 //
 //   gemm_tile    128 x 128 x 64 tiles for many rows (prefill).  Four waves, each a quarter of the
 //                tile as 2 x 2 blocks of v_mfma_f32_32x32x16_bf16; operands staged through LDS
@@ -17,14 +18,50 @@
 //
 // The weights are the MFMA "A" operand (rows = output columns n), the activations the "B"
 // operand (columns = rows m), so a lane ends up with four consecutive n of one m.
+//
+// The tile kernel's general form and the skinny kernel are templates over the element type; the
+// two leaner forms of the tile kernel are bfloat16 only.
 
 #include "host.h"
 #include "epilogue.h"
 
-#define TILE_K 64
+#define TILE_K 64            // bfloat16 values in a 128-byte row of an LDS tile
 #define TILE_ROW_BYTES 128
 
-__device__ __forceinline__ int chunks_of(int K) { return (K + 31) / 32; }
+typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
+
+// What a lane's 16-byte operand read is to the matrix cores.  bfloat16: eight K values, one
+// instruction of depth 32 (16-wide blocks; the lane's K group is lane / 16) or 16 (32-wide
+// blocks; lane / 32).  float: four K values, taken by four instructions of depth 4 (or 2), the
+// i-th multiplying element i of both operands: a lane's K group is the same for both operands,
+// so the four instructions cover 16 (or 8) distinct K values exactly once.  The result lies in
+// the lanes the same way for both types.
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+  static constexpr int ELEMS = 8;
+  static __device__ __forceinline__ void block16(floatx4& acc, int4v w, int4v a) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void block32(floatx16& acc, int4v w, int4v a) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<float> {
+  static constexpr int ELEMS = 4;
+  static __device__ __forceinline__ void block16(floatx4& acc, int4v w, int4v a) {
+    floatx4 wf = __builtin_bit_cast(floatx4, w), af = __builtin_bit_cast(floatx4, a);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[i], af[i], acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void block32(floatx16& acc, int4v w, int4v a) {
+    floatx4 wf = __builtin_bit_cast(floatx4, w), af = __builtin_bit_cast(floatx4, a);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[i], af[i], acc, 0, 0, 0);
+  }
+};
 
 // 16-byte chunk `chunk` of row `row` of an LDS tile with 128-byte rows.  LDS has 64 banks of four
 // bytes and serves 16 lanes of a 16-byte access at a time, so two rows span the banks once and
@@ -45,14 +82,16 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int blocks) {
   return xcd * q + (xcd < r ? xcd : r) + local;
 }
 
-// BM x BN x 64 tiles, WM x WN waves, each wave (BM / WM) x (BN / WN) as blocks of
-// v_mfma_f32_32x32x16_bf16; LDS holds two stages.  PF register sets hold tiles on their way
+// BM x BN tiles of 128-byte rows (64 bfloat16 or 32 float K values), WM x WN waves, each wave
+// (BM / WM) x (BN / WN) as 32-wide MFMA blocks; LDS holds two stages.  PF register sets hold tiles on their way
 // from memory to LDS: with one, the loads of tile i + 1 fly while tile i is multiplied; with
 // two, tile i + 1 waits in registers and the loads of tile i + 2 fly.
-template <int BM, int BN, int WM, int WN, int PF>
+template <typename T, int BM, int BN, int WM, int WN, int PF>
 __global__ void __launch_bounds__(WM * WN * 64)
-gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
+gemm_tile_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W, int M, int N,
                  int K, Epilogue epi, int tiles_m, int tiles_n) {
+  constexpr int ELEMS = Mma<T>::ELEMS;          // K values in a 16-byte chunk
+  constexpr int ROW_K = 8 * ELEMS;              // K values in a 128-byte row of a tile
   constexpr int THREADS = WM * WN * 64;
   constexpr int ROWS = BM + BN;                 // rows of a stage: A's, then W's
   constexpr int PER_THREAD = ROWS * 8 / THREADS;  // 16-byte chunks a thread moves per tile
@@ -66,7 +105,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
   const int tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
   const int m_base = (tile % tiles_m) * BM, n_base = (tile / tiles_m) * BN;
   const int split = blockIdx.z, splits = gridDim.z;
-  const int k_tiles = (K + TILE_K - 1) / TILE_K;
+  const int k_tiles = (K + ROW_K - 1) / ROW_K;
   const int kt_begin = (int)((int64_t)k_tiles * split / splits);
   const int kt_end = (int)((int64_t)k_tiles * (split + 1) / splits);
 
@@ -75,16 +114,15 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
   // the registers of the larger tiles.
   const int c = tid & 7, r0 = tid >> 3;
   constexpr int A_CHUNKS = BM / ROW_STEP;
-  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
   int4v regs[PF][PER_THREAD];
   auto load_tile = [&](int set, int kt) {
-    // a chunk beyond K (a multiple of 8) reads the row's last chunk and is cleared when stored
-    int k = kt * TILE_K + c * 8;
-    int kc = k < K ? k : K - 8;
+    // a chunk beyond K (a multiple of the chunk) reads the row's last chunk and is cleared when stored
+    int k = kt * ROW_K + c * ELEMS;
+    int kc = k < K ? k : K - ELEMS;
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       int row = r0 + ROW_STEP * i;
-      const bf16_t* src;
+      const T* src;
       if (i < A_CHUNKS) {
         int m = m_base + row;
         src = A + (int64_t)(m < M ? m : M - 1) * lda;
@@ -96,7 +134,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
     }
   };
   auto store_tile = [&](int set, int kt, int stage) {
-    int keep = kt * TILE_K + c * 8 < K ? -1 : 0;
+    int keep = kt * ROW_K + c * ELEMS < K ? -1 : 0;
     unsigned char* base = lds + stage * (ROWS * TILE_ROW_BYTES);
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i)
@@ -116,16 +154,16 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
     // per tile, and the reads of later steps return while earlier steps multiply
     const unsigned char* a_lds = lds + stage * (ROWS * TILE_ROW_BYTES);
     const unsigned char* w_lds = a_lds + BM * TILE_ROW_BYTES;
-    constexpr int STEPS = TILE_K / 16;
-    bf16x8 wop[STEPS][TN], aop[STEPS][TM];
+    constexpr int STEPS = TILE_ROW_BYTES / 32;      // a step: the two K groups' chunks
+    int4v wop[STEPS][TN], aop[STEPS][TM];
 #pragma unroll
     for (int kk = 0; kk < STEPS; ++kk) {
 #pragma unroll
       for (int b = 0; b < TN; ++b)
-        wop[kk][b] = *reinterpret_cast<const bf16x8*>(w_lds + swizzled(wn * (BN / WN) + b * 32 + l32, 2 * kk + g));
+        wop[kk][b] = *reinterpret_cast<const int4v*>(w_lds + swizzled(wn * (BN / WN) + b * 32 + l32, 2 * kk + g));
 #pragma unroll
       for (int b = 0; b < TM; ++b)
-        aop[kk][b] = *reinterpret_cast<const bf16x8*>(a_lds + swizzled(wm * (BM / WM) + b * 32 + l32, 2 * kk + g));
+        aop[kk][b] = *reinterpret_cast<const int4v*>(a_lds + swizzled(wm * (BM / WM) + b * 32 + l32, 2 * kk + g));
     }
 #pragma unroll
     for (int kk = 0; kk < STEPS; ++kk)
@@ -133,7 +171,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
       for (int bn = 0; bn < TN; ++bn)
 #pragma unroll
         for (int bm = 0; bm < TM; ++bm)
-          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wop[kk][bn], aop[kk][bm], acc[bn][bm], 0, 0, 0);
+          Mma<T>::block32(acc[bn][bm], wop[kk][bn], aop[kk][bm]);
   };
 
   const int count = kt_end - kt_begin;
@@ -182,7 +220,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __rest
       for (int q = 0; q < 4; ++q) {
         float v[4] = {acc[bn][bm][4 * q], acc[bn][bm][4 * q + 1], acc[bn][bm][4 * q + 2], acc[bn][bm][4 * q + 3]};
         int n0 = n_base + wn * (BN / WN) + bn * 32 + q * 8 + g * 4;
-        if (m < M) epilogue4<bf16_t>(epi, N, m, n0, v, split);
+        if (m < M) epilogue4<T>(epi, N, m, n0, v, split);
       }
     }
   }
@@ -202,7 +240,6 @@ __global__ void __launch_bounds__(256)
 gemm_tile_fast_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
                       int K, Epilogue epi, int tiles_m, int tiles_n) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * FAST_STAGE_BYTES];
-  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int wm = wave & 1, wn = wave >> 1;
   const int l32 = lane & 31, g = lane >> 5;
@@ -439,10 +476,12 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
 // MT row blocks of 16 (activations) by NT column blocks of 16 (weights) per work-group.  With
 // more than 16 rows the activations a work-group reads (all rows, its whole K range) outweigh its
 // weights, and they are read once per work-group: two column blocks halve that traffic.
-template <int MT, int NT, int U, int WAVES>
+template <typename T, int MT, int NT, int U, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
-gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
+gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W, int M, int N,
                    int K, Epilogue epi, int tile_columns) {
+  constexpr int ELEMS = Mma<T>::ELEMS;      // K values in a lane's 16-byte load
+  constexpr int CHUNK = 4 * ELEMS;          // K values the wave's four K groups cover together
   // tile_columns: how many of its 16 * NT output columns a work-group really owns (a multiple of
   // four).  Fewer than all of them is for balance: 300 work-groups of 16 columns leave 44 of 256
   // compute units with twice the bytes of the others, 400 of 12 columns leave every unit at most
@@ -456,26 +495,25 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
   const int n_base = blockIdx.x * tile_columns;
   const int n_end = n_base + tile_columns < N ? n_base + tile_columns : N;   // one past this work-group's last column
   const int split = blockIdx.y, splits = gridDim.y;
-  const bf16_t* w_row[NT];
+  const T* w_row[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     int n = n_base + nt * 16 + i16;
     w_row[nt] = W + (int64_t)(n < n_end ? n : n_end - 1) * K;
   }
-  const bf16_t* a_row[MT];
+  const T* a_row[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     int m = mt * 16 + i16;
     a_row[mt] = A + (int64_t)(m < M ? m : M - 1) * lda;
   }
-  // A batch is two phases.  First every load of the batch is issued: a chunk of 32 beyond K is
-  // skipped by a scalar branch, a group of eight beyond K (a multiple of 8) inside the last chunk
+  // A batch is two phases.  First every load of the batch is issued: a chunk beyond K is
+  // skipped by a scalar branch, a group beyond K (a multiple of the group) inside the last chunk
   // reads the row's last group instead.  Only then are the weights of such a group cleared (with
   // a bit mask) and multiplied.  Nothing that depends on a lane or on loaded data stands between
   // the loads, so the compiler has no reason to wait for one before it issues the next.
   // Rows beyond M repeat row M - 1; their results are dropped by the epilogue.
-  typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
-  const int chunks = chunks_of(K);
+  const int chunks = (K + CHUNK - 1) / CHUNK;
   const int stride = splits * WAVES;
   floatx4 acc[MT][NT];
 #pragma unroll
@@ -492,8 +530,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) av[u][mt] = int4v{0, 0, 0, 0};
       if (cc < chunks) {
-        int k = cc * 32 + g * 8;
-        int kc = k < K ? k : K - 8;
+        int k = cc * CHUNK + g * ELEMS;
+        int kc = k < K ? k : K - ELEMS;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wv[u][nt] = *reinterpret_cast<const int4v*>(w_row[nt] + kc);
 #pragma unroll
@@ -504,13 +542,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
   auto multiply = [&](int c0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      int keep = (c0 + u * stride) * 32 + g * 8 < K ? -1 : 0;
+      int keep = (c0 + u * stride) * CHUNK + g * ELEMS < K ? -1 : 0;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        bf16x8 w = __builtin_bit_cast(bf16x8, wv[u][nt] & keep);
+        int4v w = wv[u][nt] & keep;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, __builtin_bit_cast(bf16x8, av[u][mt]), acc[mt][nt], 0, 0, 0);
+        for (int mt = 0; mt < MT; ++mt) Mma<T>::block16(acc[mt][nt], w, av[u][mt]);
       }
     }
   };
@@ -541,15 +578,15 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __re
     for (int w = 0; w < WAVES; ++w)
 #pragma unroll
       for (int r = 0; r < 4; ++r) v[r] += red[w][wave][lane][r];
-    if (out_m < M) epilogue4_prefetched<bf16_t>(epi, n_end, out_m, out_n0, v, split, pre);   // nothing beyond n_end
+    if (out_m < M) epilogue4_prefetched<T>(epi, n_end, out_m, out_n0, v, split, pre);   // nothing beyond n_end
   }
 }
 
-static int check_operands(const char* who, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                          const Epilogue& e, int splits) {
+static int check_operands(const char* who, int elems, const void* A, int64_t lda, const void* W, int M, int N,
+                          int K, const Epilogue& e, int splits) {
   if (N <= 0 || K <= 0) BT_REFUSE("%s: N %d and K %d must be positive", who, N, K);
-  if (K % 8 != 0 || lda % 8 != 0)
-    BT_REFUSE("%s: K %d and the row pitch %lld must be multiples of 8 (16-byte loads)", who, K, (long long)lda);
+  if (K % elems != 0 || lda % elems != 0)
+    BT_REFUSE("%s: K %d and the row pitch %lld must be multiples of %d (16-byte loads)", who, K, (long long)lda, elems);
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) BT_REFUSE("%s: operands must be 16-byte aligned", who);
   if (e.mode < 0 || e.mode > 4 || e.out == nullptr) BT_REFUSE("%s: bad epilogue", who);
   if (splits < 1 || (splits > 1 && e.mode != EPI_F32))
@@ -566,26 +603,34 @@ static int check_operands(const char* who, const void* A, int64_t lda, const voi
   return BT_OK;
 }
 
-template <int BM, int BN, int WM, int WN, int PF>
-static void launch_tile(hipStream_t stream, const bf16_t* A, int64_t lda, const bf16_t* W, int M, int N, int K,
+template <typename T, int BM, int BN, int WM, int WN, int PF>
+static void launch_tile(hipStream_t stream, const T* A, int64_t lda, const T* W, int M, int N, int K,
                         const Epilogue& epi, int splits) {
   int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   size_t lds = (size_t)2 * (BM + BN) * TILE_ROW_BYTES;
-  auto kernel = gemm_tile_kernel<BM, BN, WM, WN, PF>;
+  auto kernel = gemm_tile_kernel<T, BM, BN, WM, WN, PF>;
   if (lds > 64 * 1024)
     (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, 1, splits), dim3(WM * WN * 64), lds, stream, A, lda, W, M, N,
                      K, epi, tiles_m, tiles_n);
 }
 
+// dtype: 0 float, 1 bfloat16 (the codes of every entry point that takes both).
 // variant: 0 = the fastest form the operands allow; 1 = template, 2 = lean, 3 = direct to LDS
-// (asked for by tests and measurements; a form that cannot take the operands is refused)
-BT_EXPORT int bt_gemm_tile_bf16(void* stream, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                                const Epilogue* epi, int splits, int variant) {
+// (asked for by tests and measurements; a form that cannot take the operands is refused; float
+// has the template only)
+BT_EXPORT int bt_gemm_tile(void* stream, int dtype, const void* A, int64_t lda, const void* W, int M, int N, int K,
+                           const Epilogue* epi, int splits, int variant) {
   if (M <= 0) return BT_OK;
-  int rc = check_operands("gemm_tile_bf16", A, lda, W, M, N, K, *epi, splits);
+  if (dtype != 0 && dtype != 1) BT_REFUSE("gemm_tile: element type %d is neither float nor bfloat16", dtype);
+  int rc = check_operands("gemm_tile", dtype == 0 ? 4 : 8, A, lda, W, M, N, K, *epi, splits);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
+  if (dtype == 0) {
+    if (variant > 1) BT_REFUSE("gemm_tile: float products have the general form only, not variant %d", variant);
+    launch_tile<float, 128, 128, 2, 2, 1>(s, (const float*)A, lda, (const float*)W, M, N, K, *epi, splits);
+    return bt_check_launch("gemm_tile");
+  }
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   const int64_t four_gib = (int64_t)1 << 32;
@@ -595,7 +640,7 @@ BT_EXPORT int bt_gemm_tile_bf16(void* stream, const void* A, int64_t lda, const 
   // work-groups per unit) when there are more.
   if (variant == 0) variant = !lean_ok ? 1 : ((int64_t)((M + 127) / 128) * ((N + 127) / 128) * splits <= 256 ? 3 : 2);
   if (variant != 1 && !lean_ok)
-    BT_REFUSE("gemm_tile_bf16: this form needs K %d to be a multiple of 64 and operands below 4 GiB", K);
+    BT_REFUSE("gemm_tile: this form needs K %d to be a multiple of 64 and operands below 4 GiB", K);
   int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
   dim3 grid(tiles_m * tiles_n, 1, splits);
   if (variant == 3) {
@@ -604,27 +649,42 @@ BT_EXPORT int bt_gemm_tile_bf16(void* stream, const void* A, int64_t lda, const 
     if (!raised) {
       hipError_t err = hipFuncSetAttribute((const void*)gemm_tile_dma_kernel,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (err != hipSuccess) BT_REFUSE("gemm_tile_bf16: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));
+      if (err != hipSuccess) BT_REFUSE("gemm_tile: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));
       raised = true;
     }
     hipLaunchKernelGGL(gemm_tile_dma_kernel, grid, dim3(256), lds, s, a, lda, w, M, N, K, *epi, tiles_m, tiles_n);
   } else if (variant == 2) {
     hipLaunchKernelGGL(gemm_tile_fast_kernel, grid, dim3(256), 0, s, a, lda, w, M, N, K, *epi, tiles_m, tiles_n);
   } else {
-    launch_tile<128, 128, 2, 2, 1>(s, a, lda, w, M, N, K, *epi, splits);
+    launch_tile<bf16_t, 128, 128, 2, 2, 1>(s, a, lda, w, M, N, K, *epi, splits);
   }
-  return bt_check_launch("gemm_tile_bf16");
+  return bt_check_launch("gemm_tile");
 }
 
-BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                                  const Epilogue* epi, int splits, int variant) {
+template <typename T>
+static void launch_skinny(hipStream_t s, const T* a, int64_t lda, const T* w, int M, int N, int K, const Epilogue& epi,
+                          int splits, int columns) {
+  dim3 grid((N + columns - 1) / columns, splits), block(512);
+#define LAUNCH_SKINNY(MT, NT, U) \
+  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns)
+  if (M <= 16) {
+    if (columns <= 16) LAUNCH_SKINNY(1, 1, 8); else LAUNCH_SKINNY(1, 2, 8);
+  } else if (M <= 32) {
+    if (columns <= 16) LAUNCH_SKINNY(2, 1, 4); else LAUNCH_SKINNY(2, 2, 4);
+  } else {
+    if (columns <= 16) LAUNCH_SKINNY(4, 1, 2); else LAUNCH_SKINNY(4, 2, 2);
+  }
+#undef LAUNCH_SKINNY
+}
+
+BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda, const void* W, int M, int N, int K,
+                             const Epilogue* epi, int splits, int variant) {
   if (M <= 0) return BT_OK;
-  if (M > 64) BT_REFUSE("gemm_skinny_bf16: %d rows, at most 64", M);
-  int rc = check_operands("gemm_skinny_bf16", A, lda, W, M, N, K, *epi, splits);
+  if (M > 64) BT_REFUSE("gemm_skinny: %d rows, at most 64", M);
+  if (dtype != 0 && dtype != 1) BT_REFUSE("gemm_skinny: element type %d is neither float nor bfloat16", dtype);
+  const int elems = dtype == 0 ? 4 : 8;
+  int rc = check_operands("gemm_skinny", elems, A, lda, W, M, N, K, *epi, splits);
   if (rc) return rc;
-  hipStream_t s = (hipStream_t)stream;
-  const bf16_t* a = (const bf16_t*)A;
-  const bf16_t* w = (const bf16_t*)W;
   // 8 to 32 columns per work-group in steps of four (one or two column blocks of the kernel),
   // whichever leaves the busiest compute unit the least to pull: work-groups land on the units in
   // whole rounds.  Variants 8, 12, ... 32 (measurements and tests) force that many.
@@ -641,7 +701,8 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
   if (variant >= 8 && variant <= 32 && variant % 4 == 0) {
     columns = variant;
   } else if (variant == 0) {
-    const int64_t per = ((K + 31) / 32 + splits - 1) / splits;
+    const int chunk = 4 * elems;
+    const int64_t per = ((K + chunk - 1) / chunk + splits - 1) / splits;
     int64_t best = -1;
     for (int c = 32; c >= 8; c -= 4) {
       int64_t groups = (int64_t)((N + c - 1) / c) * splits;
@@ -649,16 +710,9 @@ BT_EXPORT int bt_gemm_skinny_bf16(void* stream, const void* A, int64_t lda, cons
       if (best < 0 || cost < best) { best = cost; columns = c; }
     }
   }
-  dim3 grid((N + columns - 1) / columns, splits), block(512);
-#define LAUNCH_SKINNY(MT, NT, U) \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, *epi, columns)
-  if (M <= 16) {
-    if (columns <= 16) LAUNCH_SKINNY(1, 1, 8); else LAUNCH_SKINNY(1, 2, 8);
-  } else if (M <= 32) {
-    if (columns <= 16) LAUNCH_SKINNY(2, 1, 4); else LAUNCH_SKINNY(2, 2, 4);
-  } else {
-    if (columns <= 16) LAUNCH_SKINNY(4, 1, 2); else LAUNCH_SKINNY(4, 2, 2);
-  }
-#undef LAUNCH_SKINNY
-  return bt_check_launch("gemm_skinny_bf16");
+  if (dtype == 0)
+    launch_skinny<float>((hipStream_t)stream, (const float*)A, lda, (const float*)W, M, N, K, *epi, splits, columns);
+  else
+    launch_skinny<bf16_t>((hipStream_t)stream, (const bf16_t*)A, lda, (const bf16_t*)W, M, N, K, *epi, splits, columns);
+  return bt_check_launch("gemm_skinny");
 }

@@ -22,17 +22,30 @@ def _rounded(tokens):
     return (tokens + BLOCK - 1) // BLOCK * BLOCK
 
 
+def new_token_limits(prompt_lengths, max_new_tokens, total_length=None):
+    """New tokens each request may get: max_new_tokens, or fewer where prompt and output together
+    would pass ``total_length``."""
+    if total_length is None:
+        return [max_new_tokens] * len(prompt_lengths)
+    for index, length in enumerate(prompt_lengths):
+        if length >= total_length:
+            raise GenerationError(f"prompt {index} holds {length} tokens already, total_length is {total_length}")
+    return [min(max_new_tokens, total_length - length) for length in prompt_lengths]
+
+
 def plan_batches(prompt_lengths, max_new_tokens, max_tokens, max_slots, sequence_limit, batch_size=None):
     """Splits requests, in order, into batches whose sequences fit the cache together.
-    Pure bookkeeping; raises if a single request cannot fit."""
+    ``max_new_tokens`` is one number or one per request.  Pure bookkeeping; raises if a single
+    request cannot fit."""
     batches, current, used = [], [], 0
+    limits = max_new_tokens if isinstance(max_new_tokens, (list, tuple)) else [max_new_tokens] * len(prompt_lengths)
     for index, length in enumerate(prompt_lengths):
         if length <= 0:
             raise GenerationError(f"prompt {index} is empty")
-        need = required_capacity(length, max_new_tokens)
+        need = required_capacity(length, limits[index])
         if need > sequence_limit:
             raise GenerationError(
-                f"prompt {index}: {length} prompt tokens + {max_new_tokens} new tokens need {need} positions, "
+                f"prompt {index}: {length} prompt tokens + {limits[index]} new tokens need {need} positions, "
                 f"the limit is {sequence_limit}")
         if _rounded(need) > max_tokens:
             raise GenerationError(f"prompt {index} needs {_rounded(need)} cache tokens, the cache holds {max_tokens}")
@@ -60,9 +73,10 @@ def prefill_chunks(prompt_lengths, chunk):
     return steps
 
 
-def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None):
-    """Runs one batch that starts together to completion; returns its GeneratedSequences."""
-    tracker = GenerationTracker(config, [len(p) for p in prompts])
+def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None, limits=None):
+    """Runs one batch that starts together to completion; returns its GeneratedSequences.
+    ``limits``: new tokens each row may get, where that is less than config.max_new_tokens."""
+    tracker = GenerationTracker(config, [len(p) for p in prompts], limits)
     sampler = Sampler(config, len(prompts), engine.device, engine.model.vocab_size, prompts)
     slots = [engine.open() for _ in prompts]
     open_rows = set(range(len(prompts)))
@@ -102,15 +116,18 @@ def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None):
     return tracker.sequences
 
 
-def generate(engine, prompts, config=None, prefill_chunk=None, batch_size=None, on_token=None):
-    """Generates for every prompt (lists of token ids); returns GeneratedSequences in order."""
+def generate(engine, prompts, config=None, prefill_chunk=None, batch_size=None, on_token=None, total_length=None):
+    """Generates for every prompt (lists of token ids); returns GeneratedSequences in order.
+    With ``total_length`` a sequence also ends (Length) when prompt and output together hold that
+    many tokens, so unequal prompts can all be grown to the model's position limit."""
     config = config or GenerationConfig()
     config.validate(engine.model.vocab_size)
     prompts = [list(p) for p in prompts]
     if not prompts:
         raise GenerationError("no prompts")
     limit = min(engine.model.max_positions, engine.cache.max_sequence_length)
-    batches = plan_batches([len(p) for p in prompts], config.max_new_tokens, engine.cache.max_tokens,
+    limits = new_token_limits([len(p) for p in prompts], config.max_new_tokens, total_length)
+    batches = plan_batches([len(p) for p in prompts], limits, engine.cache.max_tokens,
                            engine.cache.max_slots, limit, batch_size)
     results = [None] * len(prompts)
     for batch in batches:
@@ -118,6 +135,6 @@ def generate(engine, prompts, config=None, prefill_chunk=None, batch_size=None, 
         if on_token is not None:
             callback = lambda row, token, logp, reason, batch=batch: on_token(batch[row], token, logp, reason)
         for index, sequence in zip(batch, generate_batch(engine, [prompts[i] for i in batch], config,
-                                                         prefill_chunk, callback)):
+                                                         prefill_chunk, callback, [limits[i] for i in batch])):
             results[index] = sequence
     return results

@@ -36,7 +36,7 @@ def module_source(name):
                 f"no bfloat16 attention kernel for head size {size}: "
                 f"sizes {ATTENTION_HEAD_SIZES[0]}..{ATTENTION_HEAD_SIZES[-1]} in steps of 16 are built")
         return "attention_bf16.hip", [f"-DBT_HEAD_DIM={size}"]
-    if name in ("core", "gemm_bf16"):
+    if name in ("core", "gemm_mfma", "attention_f32"):
         return name + ".hip", []
     if name == "gemm_library":      # host code around hipBLASLt, which it opens at run time
         return name + ".hip", ["-ldl"]
@@ -44,7 +44,7 @@ def module_source(name):
 
 
 def all_modules():
-    return ["core", "gemm_bf16", "gemm_library"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
+    return ["core", "gemm_mfma", "gemm_library", "attention_f32"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
 
 
 def _hash(name):

@@ -93,11 +93,13 @@ def require_gpu():
 def prepare(dtype, head_dims=()):
     """Builds and loads what a model of this dtype and these head sizes needs."""
     _module("core")
+    _module("gemm_mfma")
     if dtype == torch.bfloat16:
-        _module("gemm_bf16")
         library_products()
         for size in head_dims:
             _module(f"attention_bf16_hd{size}")
+    elif any(size <= 128 for size in head_dims):
+        _module("attention_f32")
 
 
 # --- the vendor's GEMM library for steps with many rows ---------------------------------------
@@ -158,6 +160,9 @@ def _check_library_products():
         error = float((mine.float() - theirs.float()).abs().max())
         if not error < 0.05:
             raise RuntimeError(f"its result differs from the tile kernel's by {error}")
+
+
+_library_refused = set()     # (rows, columns, k, epilogue mode, bias?) the library had no algorithm for
 
 
 def _library_takes(epilogue):
@@ -228,9 +233,9 @@ def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None,
 def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
     """C = a . w^T handed to ``epilogue``.  a: [M, K] (rows may be strided), w: [N, K] contiguous.
 
-    impl: "auto" (float32 -> plain; bfloat16 -> skinny up to 64 rows, beyond that the vendor's
-    library where it is usable and has the epilogue, else tile), or one of "plain", "tile",
-    "skinny", "library" to force one.  variant picks one of the tile kernel's forms
+    impl: "auto" (skinny up to 64 rows; beyond that the tile kernel, or for bfloat16 the vendor's
+    library where it is usable and has the epilogue; float32 operands that are not multiples of
+    four wide go to the plain kernel), or one of "plain", "tile", "skinny", "library" to force one.  variant picks one of the tile kernel's forms
     (0: the fastest the operands allow, 1: any K, 2: lean, 3: direct to LDS) or, for the skinny
     kernel, the output columns a work-group owns (8, 12, ... 32; 0: chosen for balance).
     """
@@ -240,12 +245,27 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
         raise KernelError(f"gemm: operands [{m},{k}] {a.dtype} and [{n},{w.shape[1]}] {w.dtype} do not fit")
     dtype = DTYPE_CODES[a.dtype]
     if impl == "auto":
-        if dtype == FLOAT32:
-            impl = "plain"
+        if dtype == FLOAT32 and (k % 4 or a.stride(0) % 4):
+            impl = "plain"                       # the MFMA kernels read 16 bytes at a time
         elif m <= 64:
             impl = "skinny"
+        elif dtype == FLOAT32:
+            impl = "tile"
         else:
-            impl = "library" if splits == 1 and _library_takes(epilogue) and library_products() else "tile"
+            shape = (m, n, k, int(epilogue.mode), bool(epilogue.bias))
+            impl = "library" if splits == 1 and _library_takes(epilogue) and library_products() \
+                and shape not in _library_refused else "tile"
+            if impl == "library":
+                try:
+                    gemm(a, w, epilogue, impl="library")
+                    return
+                except KernelError as refusal:      # the library has nothing for this shape: the tile kernel does
+                    if "no algorithm" not in str(refusal):
+                        raise
+                    _library_refused.add(shape)
+                    print(f"[burn_transformers_amd] {refusal}; this shape runs on the package's tile kernel",
+                          file=sys.stderr, flush=True)
+                    impl = "tile"
     args = (_c_ptr(a.data_ptr()), _c_i64(a.stride(0)), _c_ptr(w.data_ptr()), _c_int(m), _c_int(n), _c_int(k),
             ctypes.byref(epilogue))
     if impl == "plain":
@@ -254,9 +274,9 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
         lib = _module("core")
         _check(lib, lib.bt_gemm_plain(_c_ptr(_stream()), _c_int(dtype), *args))
         return
-    if dtype != BFLOAT16:
-        raise KernelError(f"gemm: the {impl} kernel takes bfloat16 only")
     if impl == "library":
+        if dtype != BFLOAT16:
+            raise KernelError("gemm: the library product takes bfloat16 only")
         lib = _library_state["lib"] or library_products()
         if lib is None:
             raise KernelError("gemm: the vendor's GEMM library is not available")
@@ -264,11 +284,9 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
             raise KernelError("gemm: the library product does not split K")
         _check(lib, lib.bt_gemm_library_bf16(_c_ptr(_stream()), *args))
         return
-    lib = _module("gemm_bf16")
-    if impl == "tile":
-        _check(lib, lib.bt_gemm_tile_bf16(_c_ptr(_stream()), *args, _c_int(splits), _c_int(variant)))
-    else:
-        _check(lib, lib.bt_gemm_skinny_bf16(_c_ptr(_stream()), *args, _c_int(splits), _c_int(variant)))
+    lib = _module("gemm_mfma")
+    entry = lib.bt_gemm_tile if impl == "tile" else lib.bt_gemm_skinny
+    _check(lib, entry(_c_ptr(_stream()), _c_int(dtype), *args, _c_int(splits), _c_int(variant)))
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
@@ -280,13 +298,24 @@ def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_head
 
 
 def attention(args, dtype, decode, impl="auto"):
-    """Attention of the step's tokens over the cache.  impl: "auto", "plain" or "mfma"."""
+    """Attention of the step's tokens over the cache.  impl: "auto" (bfloat16: the MFMA kernels;
+    float32: the tiled kernel for head sizes up to 128, else the plain one), "plain", "tiled"
+    (float32) or "mfma" (bfloat16)."""
     code = DTYPE_CODES[dtype]
     if impl == "auto":
-        impl = "plain" if code == FLOAT32 else "mfma"
+        if code == BFLOAT16:
+            impl = "mfma"
+        else:
+            impl = "tiled" if args.kv.head_dim <= 128 and args.ldq % 4 == 0 else "plain"
     if impl == "plain":
         lib = _module("core")
         _check(lib, lib.bt_attention_plain(_c_ptr(_stream()), _c_int(code), ctypes.byref(args)))
+        return
+    if impl == "tiled":
+        if code != FLOAT32:
+            raise KernelError("attention: the tiled kernel takes float32 only")
+        lib = _module("attention_f32")
+        _check(lib, lib.bt_attention_f32(_c_ptr(_stream()), ctypes.byref(args)))
         return
     if code != BFLOAT16:
         raise KernelError("attention: the MFMA kernels take bfloat16 only")

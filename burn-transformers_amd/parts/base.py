@@ -46,12 +46,17 @@ class ResidualStream:
         self.pending = delta
 
     def add_product(self, step, a, weight, bias=None):
-        """x += a . weight^T + bias.  In a bfloat16 decode step (up to 64 rows) a product with few
+        """x += a . weight^T + bias.  In a decode step (up to 64 rows) a product with few
         output columns splits its K range into partial sums that stay pending: the extra work-groups
         are needed to pull the matrix through HBM.  Otherwise the product's epilogue adds into the
         stream in place."""
         rows, width = a.shape[0], weight.shape[0]
-        splits = split_count(rows, width, a.shape[1], compute_units(a.device)) if step.dtype_is_bf16 else 1
+        if step.dtype_is_bf16:
+            splits = split_count(rows, width, a.shape[1], compute_units(a.device), 32)
+        elif a.shape[1] % 4 == 0 and a.stride(0) % 4 == 0:        # what the float32 MFMA kernels take
+            splits = split_count(rows, width, a.shape[1], compute_units(a.device), 16)
+        else:
+            splits = 1
         if splits > 1:
             partials = step.buffer("stream.partials", splits * rows, width, "float32").view(splits, rows, width)
             K.gemm(a, weight, K.epilogue_f32(partials), splits=splits)
@@ -142,12 +147,12 @@ def compute_units(device):
     return torch.cuda.get_device_properties(device).multi_processor_count
 
 
-def split_count(rows, columns, k, units=256):
+def split_count(rows, columns, k, units=256, chunk=32):
     """How many ways a residual-writing product splits its K range (up to 64 rows; 1 beyond).
 
     The skinny product gives one work-group 16 output columns (32 beyond 16 rows) and one slice
     of K, and its time is set by the compute unit that has to pull the most bytes: a unit takes a work-group of
-    ``per`` chunks of 32 in about ``per + 10`` units of time (the ten are the work-group's own
+    ``per`` chunks (``chunk`` K values: 32 of bfloat16, 16 of float32) in about ``per + 10`` units of time (the ten are the work-group's own
     start and its reduction), and ``tiles * splits`` work-groups land on ``units`` compute units
     in whole rounds.  Measured on 100 tiles: K 6400 takes 13.9 / 8.6 / 8.5 / 7.6 / 9.3 us with
     1 / 2 / 4 / 5 / 8 splits, K 1600 takes 5.0 / 4.1 / 4.2 / 4.1 / 5.2 us; the model picks 5 and 2.
@@ -155,7 +160,7 @@ def split_count(rows, columns, k, units=256):
     if rows > 64:
         return 1
     tiles = (columns + 15) // 16 if rows <= 16 else (columns + 31) // 32   # beyond 16 rows: 32 columns each
-    chunks = (k + 31) // 32
+    chunks = (k + chunk - 1) // chunk
     best, best_cost = 1, None
     for splits in range(1, 9):
         per = (chunks + splits - 1) // splits

@@ -7,6 +7,8 @@ Rules (src/generation.rs:1277-1422, src/generation/bookkeeping.rs:177-296):
     (StopSequence; ties go to the first configured); the matched tokens stay emitted;
   * otherwise reaching max_new_tokens ends it (Length);
   * before min_new_tokens neither end-of-sequence nor stop sequences are looked at.
+A sequence may have a limit of its own below max_new_tokens (a batch of unequal prompts that
+all grow to one total length); the reference has one limit for the whole batch.
 """
 
 from dataclasses import dataclass, field
@@ -36,8 +38,9 @@ class GeneratedSequence:
     finish_reason: Optional[FinishReason] = None
 
 
-def stop_decision(config, emitted):
-    """Why a sequence whose emitted tokens are ``emitted`` ends now, or None."""
+def stop_decision(config, emitted, limit=None):
+    """Why a sequence whose emitted tokens are ``emitted`` ends now, or None.  ``limit`` is the
+    sequence's own bound on new tokens where it has one (never above max_new_tokens)."""
     count = len(emitted)
     if count >= config.min_new_tokens:
         if emitted and emitted[-1] in config.eos_token_ids:
@@ -49,15 +52,16 @@ def stop_decision(config, emitted):
                 best = (index, n)
         if best is not None:
             return FinishReason("stop", index=best[0], length=best[1])
-    if count >= config.max_new_tokens:
+    if count >= (config.max_new_tokens if limit is None else min(limit, config.max_new_tokens)):
         return FinishReason("length")
     return None
 
 
 class GenerationTracker:
-    def __init__(self, config, prompt_lengths):
+    def __init__(self, config, prompt_lengths, limits=None):
         self.config = config
         self.sequences = [GeneratedSequence(n) for n in prompt_lengths]
+        self.limits = list(limits) if limits is not None else [None] * len(self.sequences)
 
     def push(self, row, token, log_probability):
         """Records a token of a live row; returns its finish reason if it ends now."""
@@ -66,7 +70,7 @@ class GenerationTracker:
             raise RuntimeError(f"row {row} has already finished")
         sequence.token_ids.append(int(token))
         sequence.log_probabilities.append(float(log_probability))
-        sequence.finish_reason = stop_decision(self.config, sequence.token_ids)
+        sequence.finish_reason = stop_decision(self.config, sequence.token_ids, self.limits[row])
         return sequence.finish_reason
 
     def finished(self, row):

@@ -62,6 +62,23 @@ def test_prompts_without_the_vendor_library(name, lengths, monkeypatch):
         engine.close(slot)
 
 
+def test_a_step_of_many_thousand_prompt_tokens():
+    """70 prompts of up to 128 tokens in one step: more rows than one call of the vendor's library
+    is given, and more sequences than a decode batch of the measured sizes."""
+    name = "A"
+    engine = engine_for(name, "bfloat16", max_tokens=70 * 128)
+    lengths = [128 - (i % 5) for i in range(70)]
+    prompts = prompts_for(name, lengths, seed=8)
+    assert sum(lengths) > 2 * 4096
+    slots = [engine.open() for _ in prompts]
+    logits = engine.step(list(zip(slots, prompts)), want=[[0, n - 1] for n in lengths]).clone()
+    for i in (0, 1, 33, 34, 68, 69):           # requests at both ends and across the runs of rows
+        check(logits[2 * i:2 * i + 2], plain_logits(name, prompts[i])[[0, lengths[i] - 1]], "bfloat16", f"request {i}")
+    for slot in slots:
+        engine.close(slot)
+    engine.cache.ledger.check()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,length", [("A", 100), ("B", 150), ("B", 33)])
 def test_last_32_tokens_one_by_one(name, dtype, length):
@@ -260,6 +277,27 @@ def test_greedy_generation_through_the_entry_point(name):
     got16 = bt.generate(engine16, prompts, bt.GenerationConfig(max_new_tokens=8))
     same = sum(a == b for s, w in zip(got16, want) for a, b in zip(s.token_ids, w))
     assert same >= 16
+    engine.cache.ledger.check()
+
+
+def test_unequal_prompts_grown_to_the_position_limit():
+    """Prompts of 5, 100 and 127 tokens all decoded to the model's 128 positions in one batch: each
+    ends by its own length, the long ones first, and the tokens are the plain greedy loop's."""
+    gain = 6.0
+    folder, config, weights = model_folder("A", gain)
+    limit = config["n_positions"]
+    prompts = prompts_for("A", [5, 100, limit - 1], seed=43)
+    engine = engine_for("A", "float32", gain=gain, max_tokens=3 * 128)
+    with pytest.raises(bt.GenerationError, match="need 204 positions, the limit is 128"):
+        bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=200))
+    order = []
+    got = bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=200), total_length=limit,
+                      on_token=lambda row, token, logp, reason: order.append(row) if reason is not None else None)
+    assert [len(s.token_ids) for s in got] == [limit - 5, limit - 100, 1]
+    assert all(str(s.finish_reason) == "Length" for s in got)
+    assert order == [2, 1, 0]
+    for prompt, sequence in zip(prompts, got):
+        assert sequence.token_ids == plain.greedy(prompt, weights, config, len(sequence.token_ids))
     engine.cache.ledger.check()
 
 

@@ -3,7 +3,7 @@
 import pytest
 
 import burn_transformers_amd as bt
-from burn_transformers_amd.engine.generate import plan_batches, prefill_chunks
+from burn_transformers_amd.engine.generate import new_token_limits, plan_batches, prefill_chunks
 from burn_transformers_amd.sampling.tracker import (GenerationTracker, required_capacity,
                                                     stop_decision)
 
@@ -153,6 +153,22 @@ def test_batches_fit_the_cache_and_follow_the_order_of_requests():
         plan_batches([130], 2, 128, 8, sequence_limit=1024)
     with pytest.raises(bt.GenerationError, match="empty"):
         plan_batches([3, 0], 2, 128, 8, 64)
+
+
+def test_limits_of_unequal_prompts_that_grow_to_one_total_length():
+    assert new_token_limits([5, 60, 63], 100, None) == [100, 100, 100]
+    assert new_token_limits([5, 60, 63], 10, total_length=64) == [10, 4, 1]
+    with pytest.raises(bt.GenerationError, match="prompt 1 holds 64 tokens already"):
+        new_token_limits([5, 64], 10, total_length=64)
+    # each request is sized by its own limit: 60 + 4 - 1 and 63 + 1 - 1 positions fit a limit of 64
+    assert plan_batches([5, 60, 63], [10, 4, 1], 10 ** 6, 8, sequence_limit=64) == [[0, 1, 2]]
+    with pytest.raises(bt.GenerationError, match="prompt 1: 60 prompt tokens \\+ 6 new tokens need 65"):
+        plan_batches([5, 60], [10, 6], 10 ** 6, 8, sequence_limit=64)
+    config = bt.GenerationConfig(max_new_tokens=5, eos_token_ids=[9])
+    tracker = GenerationTracker(config, [3, 3], limits=[2, None])
+    assert tracker.push(0, 1, -0.1) is None and tracker.push(0, 2, -0.1).kind == "length"
+    assert tracker.push(1, 1, -0.1) is None and tracker.push(1, 2, -0.1) is None
+    assert stop_decision(config, [1, 9], limit=2).kind == "eos"          # end-of-sequence still beats length
 
 
 def test_chunks_cover_every_prompt_once_and_rows_run_out():

@@ -35,7 +35,11 @@ GEMM_CASES = [("plain", "float32", 1, 50, 24), ("plain", "float32", 70, 131, 40)
               ("tile", "bfloat16", 300, 517, 1600), ("tile", "bfloat16", 65, 50257 // 16, 96),
               ("skinny", "bfloat16", 1, 100, 136), ("skinny", "bfloat16", 7, 48, 1600),
               ("skinny", "bfloat16", 16, 333, 72), ("skinny", "bfloat16", 17, 64, 320),
-              ("skinny", "bfloat16", 33, 1000, 64), ("skinny", "bfloat16", 64, 517, 6400)]
+              ("skinny", "bfloat16", 33, 1000, 64), ("skinny", "bfloat16", 64, 517, 6400),
+              ("tile", "float32", 128, 128, 32), ("tile", "float32", 200, 300, 132), ("tile", "float32", 300, 517, 1600),
+              ("tile", "float32", 65, 50257 // 16, 100), ("skinny", "float32", 1, 100, 132),
+              ("skinny", "float32", 7, 48, 1600), ("skinny", "float32", 16, 333, 76), ("skinny", "float32", 17, 64, 320),
+              ("skinny", "float32", 33, 1000, 64), ("skinny", "float32", 64, 517, 6400)]
 
 
 @pytest.mark.parametrize("impl,dtype,m,n,k", GEMM_CASES)
@@ -53,6 +57,14 @@ def test_gemm_epilogues(impl, dtype, m, n, k):
     out32 = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
     K.gemm(a, w, K.epilogue_f32(out32), impl=impl)
     assert rel_err(out32, want) < (2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k))
+    if dtype == "float32" and impl != "plain":
+        # true 32-bit products: operands with 24 significant bits whose low bits decide the sum
+        gen = torch.Generator().manual_seed(5)
+        a2 = (1.0 + torch.rand(m, k, generator=gen) * 2 ** -12).to(DEV)
+        w2 = (torch.where(torch.arange(k) % 2 == 0, 1.0, -1.0) * (1.0 + torch.rand(n, k, generator=gen) * 2 ** -12)).to(DEV)
+        want2 = a2.cpu().double() @ w2.cpu().double().t()           # sums of +-1 nearly cancel: what is left is the low bits
+        K.gemm(a2, w2, K.epilogue_f32(out32), impl=impl)
+        assert float((out32.cpu().double() - want2).abs().max()) < 1e-5 * math.sqrt(k)
 
 
 @pytest.mark.parametrize("variant", [1, 2, 3])
@@ -73,9 +85,11 @@ def test_tile_gemm_forms_agree(variant, m, n, k):
                    variant=variant)
 
 
-@pytest.mark.parametrize("m,n,k", [(65, 48, 72), (200, 300, 136), (300, 517, 1600), (2048, 1600, 320)])
+@pytest.mark.parametrize("m,n,k", [(65, 48, 72), (200, 300, 136), (300, 517, 1600), (2048, 1600, 320),
+                                   (5000, 136, 72), (32768, 96, 64)])
 def test_vendor_library_products(m, n, k):
-    """Prompt-sized products through hipBLASLt with the three epilogues it is given, against float64."""
+    """Prompt-sized products through hipBLASLt with the three epilogues it is given, against float64;
+    the tall ones go to the library in runs of rows, with and without a shorter last run."""
     if K.library_products() is None:
         pytest.skip("hipBLASLt could not be opened; the tile kernel takes these products")
     a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=m, lda=k + 8)
@@ -103,35 +117,70 @@ def test_vendor_library_products(m, n, k):
     assert torch.equal(auto, out)
 
 
+def test_a_shape_the_library_refuses_runs_on_the_tile_kernel(monkeypatch, capfd):
+    """When the library has no algorithm for a shape, "auto" says so once and takes the tile kernel."""
+    if K.library_products() is None:
+        pytest.skip("hipBLASLt could not be opened")
+    m, n, k = 130, 72, 136
+    a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=4)
+    calls = []
+
+    class Refusing:
+        def __getattr__(self, name):
+            return getattr(K._library_state["real"], name)
+
+        def bt_gemm_library_bf16(self, *args):
+            calls.append(1)
+            return 1
+
+        def bt_last_error(self):
+            return b"gemm_library: no algorithm without workspace for this test"
+
+    monkeypatch.setitem(K._library_state, "real", K._library_state["lib"])
+    monkeypatch.setitem(K._library_state, "lib", Refusing())
+    monkeypatch.setattr(K, "_library_refused", set())
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    for _ in range(2):
+        K.gemm(a, w, K.epilogue_store(out, bias))
+        assert rel_err(out, want + bias.cpu().double()) < 6e-3
+    assert len(calls) == 1                       # asked once; the refusal is remembered for the shape
+    assert "tile kernel" in capfd.readouterr().err
+
+
 @pytest.mark.parametrize("m,n,k,splits", [(1, 100, 136, 1), (8, 4800, 1600, 2), (16, 1600, 1600, 4),
                                           (7, 333, 6400, 8), (3, 50, 1760, 1), (16, 517, 1608, 3),
                                           (2, 16, 8, 1), (9, 40, 3400, 1)])
 @pytest.mark.parametrize("columns", [0, 16, 12, 8, 20, 28, 32])
-def test_skinny_gemm_at_decode_sizes(m, n, k, splits, columns):
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_skinny_gemm_at_decode_sizes(m, n, k, splits, columns, dtype):
     """Up to 16 rows, K with a short last chunk, slices of K that do not divide evenly; 16, 12 or 8
     to 32 output columns per work-group (0: chosen for balance)."""
     variant = columns
-    a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=k, lda=k + 24)
+    dt = DTYPES[dtype]
+    a, w, bias, want = operands(m, n, k, dt, seed=k, lda=k + 24)
     parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
     K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl="skinny", variant=variant)
-    assert rel_err(parts.sum(0), want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
+    assert rel_err(parts.sum(0), want + bias.cpu().double()) < (2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k))
     if splits == 1:
-        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        out = torch.full((m, n), float("nan"), dtype=dt, device=DEV)
         K.gemm(a, w, K.epilogue_act(out, "gelu_tanh", bias), impl="skinny", variant=variant)
-        assert rel_err(out, gelu_tanh(want + bias.cpu().double())) < 6e-3
+        assert rel_err(out, gelu_tanh(want + bias.cpu().double())) < (2e-6 if dtype == "float32" else 6e-3)
 
 
 @pytest.mark.parametrize("impl,m,n,k,splits", [("skinny", 5, 96, 1600, 4), ("skinny", 64, 50, 6400, 8),
                                                ("skinny", 20, 1600, 320, 2), ("tile", 150, 200, 1600, 3)])
-def test_gemm_split_k_partials(impl, m, n, k, splits):
-    a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=splits)
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_gemm_split_k_partials(impl, m, n, k, splits, dtype):
+    a, w, bias, want = operands(m, n, k, DTYPES[dtype], seed=splits)
     parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
     K.gemm(a, w, K.epilogue_f32(parts, bias), splits=splits, impl=impl)
-    assert rel_err(parts.sum(0), want + bias.cpu().double()) < 2e-5 * math.sqrt(k)
+    assert rel_err(parts.sum(0), want + bias.cpu().double()) < (2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k))
 
 
 @pytest.mark.parametrize("impl,dtype,m,n,k", [("plain", "float32", 9, 50, 24), ("tile", "bfloat16", 130, 96, 200),
-                                               ("skinny", "bfloat16", 8, 1600, 6400), ("skinny", "bfloat16", 3, 40, 96)])
+                                               ("skinny", "bfloat16", 8, 1600, 6400), ("skinny", "bfloat16", 3, 40, 96),
+                                               ("tile", "float32", 130, 96, 200), ("skinny", "float32", 8, 1600, 6400),
+                                               ("skinny", "float32", 3, 40, 100)])
 def test_gemm_adds_into_the_residual_stream(impl, dtype, m, n, k):
     a, w, bias, want = operands(m, n, k, DTYPES[dtype], seed=77)
     gen = torch.Generator().manual_seed(1)
@@ -153,11 +202,21 @@ def test_gemm_refuses_what_it_cannot_take():
         K.gemm(a, w, K.epilogue_store(out), impl="skinny")
     with pytest.raises(K.KernelError, match="partial sums"):
         K.gemm(a, w, K.epilogue_store(out), impl="tile", splits=2)
+    a, w, bias, _ = operands(4, 32, 18, torch.float32)
+    out = torch.empty(4, 32, dtype=torch.float32, device=DEV)
+    with pytest.raises(K.KernelError, match="multiples of 4"):
+        K.gemm(a, w, K.epilogue_store(out), impl="skinny")
+    K.gemm(a, w, K.epilogue_store(out))                       # "auto" gives such float32 operands to the plain kernel
+    assert rel_err(out, a.cpu().double() @ w.cpu().double().t()) < 2e-6
+    with pytest.raises(K.KernelError, match="general form only"):
+        a, w, bias, _ = operands(128, 128, 64, torch.float32)
+        K.gemm(a, w, K.epilogue_store(torch.empty(128, 128, device=DEV)), impl="tile", variant=2)
 
 
 @pytest.mark.parametrize("impl,dtype,counts", [("plain", "float32", [3, 1, 70]), ("plain", "bfloat16", [5, 2]),
                                                ("tile", "bfloat16", [100, 1, 37]), ("skinny", "bfloat16", [1, 1, 1]),
-                                               ("skinny", "bfloat16", [9, 30])])
+                                               ("skinny", "bfloat16", [9, 30]), ("tile", "float32", [100, 1, 37]),
+                                               ("skinny", "float32", [1, 1, 1]), ("skinny", "float32", [9, 30])])
 def test_fused_projection_scatters_into_the_cache(impl, dtype, counts):
     dt = DTYPES[dtype]
     q_heads, kv_heads, hd, width = 4, 2, 32, 72
@@ -210,6 +269,33 @@ def test_attention_plain(dtype, q_heads, kv_heads, hd, totals, counts, window):
     K.attention(args, dt, decode=max(counts) == 1, impl="plain")
     want = case.reference(q, q_heads, scale, window)
     assert rel_err(out, want) < (3e-6 if dtype == "float32" else 8e-3)
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,hd,totals,counts,window",
+                         ATTN_CASES + [(2, 1, 112, [500, 64, 1], [500, 33, 1], 0), (1, 1, 96, [130], [70], 33)])
+def test_attention_tiled_float32(q_heads, kv_heads, hd, totals, counts, window):
+    """The float path's tiled kernel: prompts, chunks and single tokens through the same code; a
+    query's result is bitwise the same whether it comes alone or among others."""
+    dt = torch.float32
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=2, poison=True)
+    gen = torch.Generator().manual_seed(5)
+    q = torch.randn(case.n_tokens, q_heads * hd, generator=gen).to(DEV)
+    out = torch.full((case.n_tokens, q_heads * hd), float("nan"), dtype=dt, device=DEV)
+    scale = 0.37 / math.sqrt(hd)
+    args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                            q_heads, len(totals), max(counts), scale, window)
+    K.attention(args, dt, decode=max(counts) == 1, impl="tiled")
+    want = case.reference(q, q_heads, scale, window)
+    assert rel_err(out, want) < 3e-6
+    # the last token of every sequence alone, as a decode step would bring it
+    last = [int(case.seq_off[i + 1]) - 1 for i in range(len(totals))]
+    alone = PagedCase(totals, [1] * len(totals), kv_heads, hd, dt, DEV, seed=2, poison=True)
+    q1 = q[last].contiguous()
+    out1 = torch.full((len(totals), q_heads * hd), float("nan"), dtype=dt, device=DEV)
+    args = K.attention_args(q1, out1, alone.view(), alone.tok_seq, alone.tok_pos, alone.seq_off, alone.seq_start,
+                            q_heads, len(totals), 1, scale, window)
+    K.attention(args, dt, decode=True, impl="tiled")
+    assert torch.equal(out1, out[last])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -267,9 +353,8 @@ def test_attention_mfma(q_heads, kv_heads, hd, totals, counts, window):
 
 def test_attention_finds_one_far_key_among_hundreds():
     """One key far back is made to dominate; an off-by-one in block or tile addressing loses it."""
-    dt = torch.bfloat16
     hd, total = 64, 700
-    for target in (0, 63, 64, 333, 698):
+    for dt, target in [(torch.bfloat16, t) for t in (0, 63, 64, 333, 698)] + [(torch.float32, t) for t in (0, 64, 333, 698)]:
         case = PagedCase([total], [1], 1, hd, dt, DEV, seed=target)
         q = torch.zeros(1, hd)
         q[0, 3] = 8.0
@@ -281,7 +366,8 @@ def test_attention_finds_one_far_key_among_hundreds():
         q = q.to(dt).to(DEV)
         want = case.reference(q, 1, 1.0)
         assert (want[0] - case.v_rows[0][target].double()).abs().max() < 1e-3
-        for impl, decode in (("plain", True), ("mfma", True), ("mfma", False)):
+        impls = (("plain", True), ("mfma", True), ("mfma", False)) if dt == torch.bfloat16 else (("plain", True), ("tiled", True))
+        for impl, decode in impls:
             out = torch.empty(1, hd, dtype=dt, device=DEV)
             args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
                                     1, 1, 1, 1.0, 0)

@@ -4,7 +4,13 @@ Parameters: width, inner, activation ("gelu_tanh": 0.5x(1+tanh(sqrt(2/pi)(x+0.04
 "gelu_erf": x(1+erf(x/sqrt 2))/2; src/feed_forward.rs:351-387).  The activation runs in 32-bit
 inside the up projection's epilogue (src/feed_forward.rs:397-406 widens half inputs too); the
 down projection adds into the residual stream.
+
+The MFMA kernels read operands 16 bytes at a time, so an inner width that is no multiple of 8 is
+padded once, when the part is built: zero rows (and zero bias) in the up projection give
+act(0) = 0 in the padded columns, which meet zero columns of the down projection.
 """
+
+import torch
 
 from ..kernels import library as K
 from .base import FeedForward
@@ -25,9 +31,17 @@ class DenseFeedForward(FeedForward):
             raise ValueError(f"feed-forward: projections are {tuple(self.up_weight.shape)} and "
                              f"{tuple(self.down_weight.shape)}, expected {(self.inner, self.width)} and "
                              f"{(self.width, self.inner)}")
+        self.padded = (self.inner + 7) // 8 * 8
+        extra = self.padded - self.inner
+        if extra:
+            up, down = self.up_weight, self.down_weight
+            self.up_weight = torch.cat([up, up.new_zeros(extra, self.width)]).contiguous()
+            self.down_weight = torch.cat([down, down.new_zeros(self.width, extra)], dim=1).contiguous()
+            if self.up_bias is not None:
+                self.up_bias = torch.cat([self.up_bias, self.up_bias.new_zeros(extra)]).contiguous()
 
     def forward(self, h, step, stream):
         tokens = h.shape[0]
-        hidden = step.buffer("feed_forward.hidden", tokens, self.inner, step.dtype)
+        hidden = step.buffer("feed_forward.hidden", tokens, self.padded, step.dtype)
         K.gemm(h, self.up_weight, K.epilogue_act(hidden, self.activation, self.up_bias))
         stream.add_product(step, hidden, self.down_weight, self.down_bias)

@@ -16,7 +16,11 @@ TINY_A = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer":
 TINY_B = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 3, "n_embd": 96, "n_head": 2,
           "n_inner": 320, "vocab_size": 517, "n_positions": 192, "activation_function": "gelu",
           "layer_norm_epsilon": 1e-6, "scale_attn_by_inverse_layer_idx": True}
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1)}
+# an inner width that is odd, one head size, one layer: sizes the 16-byte loads of the kernels do not divide
+TINY_C = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 1, "n_embd": 32, "n_head": 2,
+          "n_inner": 37, "vocab_size": 131, "n_positions": 80, "activation_function": "gelu_new",
+          "layer_norm_epsilon": 1e-3, "scale_attn_by_inverse_layer_idx": False}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
 
 _folders = {}
 

@@ -30,7 +30,7 @@ def check(got, want, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,lengths", [("A", [5, 11, 17, 100]), ("B", [1, 23, 64, 65, 150])])
+@pytest.mark.parametrize("name,lengths", [("A", [5, 11, 17, 100]), ("B", [1, 23, 64, 65, 150]), ("C", [3, 80])])
 def test_each_request_alone_and_whole(name, dtype, lengths):
     engine = engine_for(name, dtype)
     for ids in prompts_for(name, lengths):
@@ -80,7 +80,7 @@ def test_a_step_of_many_thousand_prompt_tokens():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,length", [("A", 100), ("B", 150), ("B", 33)])
+@pytest.mark.parametrize("name,length", [("A", 100), ("B", 150), ("B", 33), ("C", 70)])
 def test_last_32_tokens_one_by_one(name, dtype, length):
     engine = engine_for(name, dtype)
     ids = prompts_for(name, [length], seed=3)[0]

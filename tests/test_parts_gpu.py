@@ -61,7 +61,8 @@ def test_norm_adds_what_is_pending_then_normalises(kind, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("width,inner,activation,tokens", [(80, 200, "gelu_erf", 5), (48, 72, "gelu_tanh", 70)])
+@pytest.mark.parametrize("width,inner,activation,tokens", [(80, 200, "gelu_erf", 5), (48, 72, "gelu_tanh", 70),
+                                                           (64, 100, "gelu_tanh", 3), (48, 37, "gelu_erf", 70)])
 def test_dense_feed_forward_alone(dtype, width, inner, activation, tokens):
     gen, dt = torch.Generator().manual_seed(2), DTYPES[dtype]
     up, down = rnd(gen, inner, width, scale=width ** -0.5).to(dt), rnd(gen, width, inner, scale=inner ** -0.5).to(dt)

@@ -160,7 +160,7 @@ def main():
             points[f"decode_b{batch}"] = round(batch * s / e, 1)
 
     print(json.dumps({
-        "metric": "decode tok/s at batch 8 (GPT-2 XL sizes, 512-token prompts decoded to 1,024)",
+        "metric": f"decode tok/s at batch {args.batch} (GPT-2 XL sizes, 512-token prompts decoded to 1,024)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic token ids, random weights",

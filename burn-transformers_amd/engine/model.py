@@ -70,14 +70,15 @@ class CausalLM:
     def forward(self, step, cache, readout=True):
         """Logits (float32 [len(step.sel_rows), vocab]) of the step's wanted rows; with
         ``readout=False`` the layers only fill the cache and nothing is returned."""
-        stream = self.embedding.embed(step)
-        for entry in self.schedule:
-            memory = Memory(cache, entry.cache, entry.writes, step) if entry.cache is not None else None
-            self.blocks[entry.layer].forward(stream, step, memory)
-        if not readout:
-            return None
-        hidden = self.final_norm.apply(stream, step, rows=step.sel_rows)
-        return self.readout.logits(hidden, step)
+        with K.one_stream():          # the hundreds of launches below ask for the current stream once
+            stream = self.embedding.embed(step)
+            for entry in self.schedule:
+                memory = Memory(cache, entry.cache, entry.writes, step) if entry.cache is not None else None
+                self.blocks[entry.layer].forward(stream, step, memory)
+            if not readout:
+                return None
+            hidden = self.final_norm.apply(stream, step, rows=step.sel_rows)
+            return self.readout.logits(hidden, step)
 
 
 def _device(device):

@@ -88,8 +88,13 @@ class BufferPool:
 
     def __init__(self, device):
         self.device, self.buffers, self.generation, self.frozen = device, {}, 0, False
+        self.views = {}         # (key, dtype, rows, cols) -> the view handed out last time: a step asks hundreds of times
 
     def take(self, key, rows, cols, dtype):
+        view = self.views.get((key, dtype, rows, cols))
+        if view is not None:
+            return view
+        asked = dtype
         if isinstance(dtype, str):
             dtype = getattr(torch, dtype)
         need = rows * cols
@@ -99,9 +104,14 @@ class BufferPool:
                 raise RuntimeError(f"workspace {key!r} would have to grow while a graph is being captured")
             if held is not None:
                 self.generation += 1
+                self.views = {k: v for k, v in self.views.items() if k[0] != key}      # they show the old memory
             held = torch.empty(max(need, 1), dtype=dtype, device=self.device)
             self.buffers[(key, dtype)] = held
-        return held[:need].view(rows, cols)
+        view = held[:need].view(rows, cols)
+        if len(self.views) > 4096:
+            self.views.clear()
+        self.views[(key, asked, rows, cols)] = view
+        return view
 
     def bytes(self):
         return sum(t.numel() * t.element_size() for t in self.buffers.values())

@@ -54,6 +54,9 @@ _lock = threading.Lock()
 
 
 def _module(name):
+    lib = _modules.get(name)          # (a dict read is atomic; the lock is for building and loading)
+    if lib is not None:
+        return lib
     with _lock:
         lib = _modules.get(name)
         if lib is None:
@@ -72,8 +75,28 @@ def _check(lib, code):
         raise KernelError(lib.bt_last_error().decode())
 
 
+_held_stream = [None]
+
+
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    held = _held_stream[0]
+    return held if held is not None else torch.cuda.current_stream().cuda_stream
+
+
+class one_stream:
+    """While this context is open every kernel goes to the stream that was current when it was
+    entered, looked up once: asking torch for the current stream costs more host time than a launch
+    does, and a step is hundreds of launches.  Enter it inside whatever chose the stream (a
+    ``torch.cuda.stream`` or ``torch.cuda.graph`` context), never around it."""
+
+    def __enter__(self):
+        self.before = _held_stream[0]
+        _held_stream[0] = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        _held_stream[0] = self.before
+        return False
 
 
 def _ptr(tensor):

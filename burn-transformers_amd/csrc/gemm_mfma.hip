@@ -476,12 +476,35 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
 // MT row blocks of 16 (activations) by NT column blocks of 16 (weights) per work-group.  With
 // more than 16 rows the activations a work-group reads (all rows, its whole K range) outweigh its
 // weights, and they are read once per work-group: two column blocks halve that traffic.
-template <typename T, int MT, int NT, int U, int WAVES>
+//
+// QPL > 0 (bfloat16, up to 16 rows): the activations are not read from memory but made here, as
+// the normalised rows of the float32 residual stream (NormOperand): the norm that would
+// otherwise be a kernel of its own in front of this one.  Every work-group normalises all rows
+// (a wave takes rows w and w + 8: the row in its registers, QPL quads of four floats per lane,
+// statistics as wave reductions) and leaves them in LDS as bfloat16, where the multiplication
+// reads its operand.  The rows' loads are issued before the first batch of weights, so the
+// statistics are computed while the weights are on their way.
+struct NormOperand {
+  const float* x;        // [M][ldx] float32 rows
+  int64_t ldx;
+  const float* gamma;    // [K]
+  const float* beta;     // [K] or null
+  float eps;
+  int kind;              // 0: layer norm, 1: RMS norm
+};
+
+__device__ float bt_norm_zeros[4] = {0.f, 0.f, 0.f, 0.f};
+
+template <typename T, int MT, int NT, int U, int WAVES, int QPL = 0>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W, int M, int N,
-                   int K, Epilogue epi, int tile_columns) {
+                   int K, Epilogue epi, int tile_columns, NormOperand norm) {
   constexpr int ELEMS = Mma<T>::ELEMS;      // K values in a lane's 16-byte load
   constexpr int CHUNK = 4 * ELEMS;          // K values the wave's four K groups cover together
+  constexpr bool NORM = QPL > 0;
+  static_assert(!NORM || (MT == 1 && sizeof(T) == 2), "the fused norm is for bfloat16 and up to 16 rows");
+  extern __shared__ __attribute__((aligned(16))) unsigned char normed[];   // NORM: [16][K * 2 + 16] bytes
+  const int normed_pitch = K * 2 + 16;      // the 16 bytes spread the rows over the LDS banks
   // tile_columns: how many of its 16 * NT output columns a work-group really owns (a multiple of
   // four).  Fewer than all of them is for balance: 300 work-groups of 16 columns leave 44 of 256
   // compute units with twice the bytes of the others, 400 of 12 columns leave every unit at most
@@ -534,8 +557,10 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
         int kc = k < K ? k : K - ELEMS;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wv[u][nt] = *reinterpret_cast<const int4v*>(w_row[nt] + kc);
+        if constexpr (!NORM) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + kc);
+          for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + kc);
+        }
       }
     }
   };
@@ -551,8 +576,79 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
       }
     }
   };
+  // NORM: the operand of every chunk of the batch from LDS (a chunk beyond K reads the row's last
+  // group, as the loads from memory do; its weights are cleared)
+  auto operands_from_lds = [&](int c0) {
+    const int row = i16 < M ? i16 : M - 1;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int k = (c0 + u * stride) * CHUNK + g * ELEMS;
+      int kc = k < K ? k : K - ELEMS;
+      av[u][0] = *reinterpret_cast<const int4v*>(normed + row * normed_pitch + kc * 2);
+    }
+  };
   int c0 = split * WAVES + wave;
-  issue(c0);
+  if constexpr (NORM) {
+    const int quads = K >> 2;
+    const float4* g4 = reinterpret_cast<const float4*>(norm.gamma);
+    const float4* b4 = reinterpret_cast<const float4*>(norm.beta);
+    const float4* z4 = reinterpret_cast<const float4*>(bt_norm_zeros);
+    float4 xv[QPL], gv[QPL], bv[QPL];
+    auto load_row = [&](int r) {
+      const float4* xr = reinterpret_cast<const float4*>(norm.x + (int64_t)r * norm.ldx);
+#pragma unroll
+      for (int q = 0; q < QPL; ++q) {
+        int c = lane + 64 * q;
+        int cc = c < quads ? c : 0;          // lanes beyond the row read its start; the result is never used
+        xv[q] = xr[cc];
+        gv[q] = g4[cc];
+        bv[q] = norm.beta ? b4[cc] : z4[0];
+      }
+    };
+    auto normalise_row = [&](int r) {
+      float part = 0.f;
+#pragma unroll
+      for (int q = 0; q < QPL; ++q)
+        if (lane + 64 * q < quads)
+          part += norm.kind == 0 ? (xv[q].x + xv[q].y + xv[q].z + xv[q].w)
+                                 : (xv[q].x * xv[q].x + xv[q].y * xv[q].y + xv[q].z * xv[q].z + xv[q].w * xv[q].w);
+      float total = wave_sum(part);
+      float mean = 0.f, rstd;
+      if (norm.kind == 0) {
+        mean = total / (float)K;
+        float sq = 0.f;
+#pragma unroll
+        for (int q = 0; q < QPL; ++q)
+          if (lane + 64 * q < quads) {
+            float a0 = xv[q].x - mean, a1 = xv[q].y - mean, a2 = xv[q].z - mean, a3 = xv[q].w - mean;
+            sq += a0 * a0 + a1 * a1 + a2 * a2 + a3 * a3;
+          }
+        rstd = 1.0f / sqrtf(wave_sum(sq) / (float)K + norm.eps);
+      } else {
+        rstd = 1.0f / sqrtf(total / (float)K + norm.eps);
+      }
+#pragma unroll
+      for (int q = 0; q < QPL; ++q) {
+        int c = lane + 64 * q;
+        if (c < quads) {
+          bf16x4 y = {(bf16_t)((xv[q].x - mean) * rstd * gv[q].x + bv[q].x), (bf16_t)((xv[q].y - mean) * rstd * gv[q].y + bv[q].y),
+                      (bf16_t)((xv[q].z - mean) * rstd * gv[q].z + bv[q].z), (bf16_t)((xv[q].w - mean) * rstd * gv[q].w + bv[q].w)};
+          *reinterpret_cast<bf16x4*>(normed + r * normed_pitch + c * 8) = y;
+        }
+      }
+    };
+    if (wave < M) load_row(wave);            // (the wave's number is scalar: no lane-dependent branch)
+    issue(c0);                               // the weights of the first batch, behind the row
+    if (wave < M) normalise_row(wave);
+    if (wave + WAVES < M) {
+      load_row(wave + WAVES);
+      normalise_row(wave + WAVES);
+    }
+    __syncthreads();
+    operands_from_lds(c0);
+  } else {
+    issue(c0);
+  }
   // wave w < MT * NT finishes row block w / NT of column block w % NT: lane holds D[i][j],
   // i = 4 * (lane / 16) + r (column n), j = lane % 16 (row m); what its epilogue needs is
   // fetched now, behind the first batch
@@ -564,6 +660,7 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
   multiply(c0);
   for (c0 += stride * U; c0 < chunks; c0 += stride * U) {
     issue(c0);
+    if constexpr (NORM) operands_from_lds(c0);
     multiply(c0);
   }
 #pragma unroll
@@ -665,8 +762,9 @@ template <typename T>
 static void launch_skinny(hipStream_t s, const T* a, int64_t lda, const T* w, int M, int N, int K, const Epilogue& epi,
                           int splits, int columns) {
   dim3 grid((N + columns - 1) / columns, splits), block(512);
+  const NormOperand none = {};
 #define LAUNCH_SKINNY(MT, NT, U) \
-  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns)
+  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns, none)
   if (M <= 16) {
     if (columns <= 16) LAUNCH_SKINNY(1, 1, 8); else LAUNCH_SKINNY(1, 2, 8);
   } else if (M <= 32) {
@@ -677,12 +775,48 @@ static void launch_skinny(hipStream_t s, const T* a, int64_t lda, const T* w, in
 #undef LAUNCH_SKINNY
 }
 
+// The product of the normalised rows of a float32 residual stream (see NormOperand): bfloat16
+// weights, up to 16 rows, K up to 2048 and a multiple of 8.
+static int launch_skinny_norm(hipStream_t s, const NormOperand& norm, const bf16_t* w, int M, int N, int K,
+                              const Epilogue& epi, int splits, int columns) {
+  dim3 grid((N + columns - 1) / columns, splits), block(512);
+  size_t lds = (size_t)16 * (K * 2 + 16);
+#define LAUNCH_NORM(NT, QPL)                                                                                   \
+  do {                                                                                                         \
+    auto kernel = gemm_skinny_kernel<bf16_t, 1, NT, 8, 8, QPL>;                                                \
+    static size_t granted = 0;    /* statically allocated LDS comes on top: ask for room beyond the default */ \
+    if (lds > granted) {                                                                                       \
+      hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (err != hipSuccess) BT_REFUSE("gemm_skinny: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));   \
+      granted = lds;                                                                                           \
+    }                                                                                                          \
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)nullptr, (int64_t)0, w, M, N, K, epi, columns, norm); \
+  } while (0)
+  if (K <= 1024) {
+    if (columns <= 16) LAUNCH_NORM(1, 4); else LAUNCH_NORM(2, 4);
+  } else {
+    if (columns <= 16) LAUNCH_NORM(1, 8); else LAUNCH_NORM(2, 8);
+  }
+#undef LAUNCH_NORM
+  return BT_OK;
+}
+
+// norm: null, or the activations are the normalised rows it describes (then A and lda are ignored)
 BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                             const Epilogue* epi, int splits, int variant) {
+                             const Epilogue* epi, int splits, int variant, const NormOperand* norm) {
   if (M <= 0) return BT_OK;
   if (M > 64) BT_REFUSE("gemm_skinny: %d rows, at most 64", M);
   if (dtype != 0 && dtype != 1) BT_REFUSE("gemm_skinny: element type %d is neither float nor bfloat16", dtype);
   const int elems = dtype == 0 ? 4 : 8;
+  if (norm != nullptr) {
+    if (dtype != 1 || M > 16 || K > 2048)
+      BT_REFUSE("gemm_skinny: the fused norm takes bfloat16 weights, up to 16 rows and K up to 2048 (got %d rows, K %d)", M, K);
+    if (!norm->x || !norm->gamma || norm->ldx < K || norm->ldx % 4 != 0 || ((uintptr_t)norm->x & 15) ||
+        ((uintptr_t)norm->gamma & 15) || ((uintptr_t)norm->beta & 15) || (norm->kind != 0 && norm->kind != 1))
+      BT_REFUSE("gemm_skinny: the rows to normalise, their scale and shift must be 16-byte aligned float32");
+    A = W;            // (only its alignment is looked at below)
+    lda = K;
+  }
   int rc = check_operands("gemm_skinny", elems, A, lda, W, M, N, K, *epi, splits);
   if (rc) return rc;
   // 8 to 32 columns per work-group in steps of four (one or two column blocks of the kernel),
@@ -710,9 +844,13 @@ BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda
       if (best < 0 || cost < best) { best = cost; columns = c; }
     }
   }
-  if (dtype == 0)
+  if (norm != nullptr) {
+    rc = launch_skinny_norm((hipStream_t)stream, *norm, (const bf16_t*)W, M, N, K, *epi, splits, columns);
+    if (rc) return rc;
+  } else if (dtype == 0) {
     launch_skinny<float>((hipStream_t)stream, (const float*)A, lda, (const float*)W, M, N, K, *epi, splits, columns);
-  else
+  } else {
     launch_skinny<bf16_t>((hipStream_t)stream, (const bf16_t*)A, lda, (const bf16_t*)W, M, N, K, *epi, splits, columns);
+  }
   return bt_check_launch("gemm_skinny");
 }

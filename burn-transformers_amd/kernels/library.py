@@ -49,6 +49,29 @@ class AttnArgs(ctypes.Structure):
                 ("max_count", _c_int), ("window", _c_int), ("scale", _c_float)]
 
 
+class NormOperand(ctypes.Structure):
+    _fields_ = [("x", _c_ptr), ("ldx", _c_i64), ("gamma", _c_ptr), ("beta", _c_ptr), ("eps", _c_float),
+                ("kind", _c_int)]
+
+
+class Normalized:
+    """Rows of the float32 residual stream that are still to be normalised: handed to ``gemm`` in
+    place of its activations, the skinny product kernel normalises them itself (up to 16 rows of
+    bfloat16 products, width up to 2048), which saves the norm's own kernel in front of it."""
+
+    MAX_ROWS, MAX_WIDTH = 16, 2048
+
+    def __init__(self, x, gamma, beta, eps, kind):
+        self.x, self.gamma, self.beta, self.eps, self.kind = x, gamma, beta, eps, kind
+        self.shape = x.shape
+        self.dtype = torch.bfloat16
+        self.device = x.device
+
+    @classmethod
+    def possible(cls, rows, width):
+        return rows <= cls.MAX_ROWS and width <= cls.MAX_WIDTH and width % 8 == 0
+
+
 _modules = {}
 _lock = threading.Lock()
 
@@ -264,6 +287,16 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
     """
     m, k = a.shape
     n = w.shape[0]
+    if isinstance(a, Normalized):
+        if w.shape[1] != k or not w.is_contiguous() or w.dtype != torch.bfloat16 or impl not in ("auto", "skinny"):
+            raise KernelError(f"gemm: rows to be normalised [{m},{k}] go with bfloat16 weights [{n},{k}] on the skinny kernel only")
+        operand = NormOperand(x=a.x.data_ptr(), ldx=a.x.stride(0), gamma=a.gamma.data_ptr(), beta=_ptr(a.beta),
+                              eps=a.eps, kind=NORM_KINDS[a.kind])
+        lib = _module("gemm_mfma")
+        _check(lib, lib.bt_gemm_skinny(_c_ptr(_stream()), _c_int(BFLOAT16), None, _c_i64(0), _c_ptr(w.data_ptr()),
+                                       _c_int(m), _c_int(n), _c_int(k), ctypes.byref(epilogue), _c_int(splits),
+                                       _c_int(variant), ctypes.byref(operand)))
+        return
     if w.shape[1] != k or a.stride(1) != 1 or not w.is_contiguous() or a.dtype != w.dtype:
         raise KernelError(f"gemm: operands [{m},{k}] {a.dtype} and [{n},{w.shape[1]}] {w.dtype} do not fit")
     dtype = DTYPE_CODES[a.dtype]
@@ -308,8 +341,10 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
         _check(lib, lib.bt_gemm_library_bf16(_c_ptr(_stream()), *args))
         return
     lib = _module("gemm_mfma")
-    entry = lib.bt_gemm_tile if impl == "tile" else lib.bt_gemm_skinny
-    _check(lib, entry(_c_ptr(_stream()), _c_int(dtype), *args, _c_int(splits), _c_int(variant)))
+    if impl == "tile":
+        _check(lib, lib.bt_gemm_tile(_c_ptr(_stream()), _c_int(dtype), *args, _c_int(splits), _c_int(variant)))
+    else:
+        _check(lib, lib.bt_gemm_skinny(_c_ptr(_stream()), _c_int(dtype), *args, _c_int(splits), _c_int(variant), None))
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,

@@ -39,6 +39,9 @@ class ResidualStream:
     def __init__(self, x):
         self.x = x              # float32 [tokens, width]
         self.pending = None     # Delta or None
+        # set by a block around a part whose output the next norm wants in the stream itself, not
+        # pending beside it (the norm is then folded into the product that follows it)
+        self.in_place = False
 
     def add(self, delta):
         if self.pending is not None:
@@ -51,7 +54,9 @@ class ResidualStream:
         are needed to pull the matrix through HBM.  Otherwise the product's epilogue adds into the
         stream in place."""
         rows, width = a.shape[0], weight.shape[0]
-        if step.dtype_is_bf16:
+        if self.in_place:
+            splits = 1
+        elif step.dtype_is_bf16:
             splits = split_count(rows, width, a.shape[1], compute_units(a.device), 32)
         elif a.shape[1] % 4 == 0 and a.stride(0) % 4 == 0:        # what the float32 MFMA kernels take
             splits = split_count(rows, width, a.shape[1], compute_units(a.device), 16)
@@ -97,6 +102,12 @@ class Norm(Part):
         """Normalised rows as a tensor [rows, width] in the step's dtype."""
         raise NotImplementedError
 
+    def deferred(self, stream, step):
+        """The stream's rows as an operand that the next product normalises itself
+        (``kernels.library.Normalized``), or None where this norm, this step or what is pending on
+        the stream does not allow it; the caller then calls ``apply``."""
+        return None
+
 
 class Mixer(Part):
     # False for a mixer whose forward reads the step's host tables (``step.host``) or otherwise
@@ -119,6 +130,10 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    # True for a feed-forward that hands ``h`` to ``kernels.library.gemm`` and looks at nothing
+    # but its shape: it may then get rows that are still to be normalised (Norm.deferred)
+    takes_deferred_norm = False
+
     def forward(self, h, step, stream):
         """Adds the feed-forward's contribution to ``stream`` (or returns it as a Delta)."""
         raise NotImplementedError

@@ -19,6 +19,8 @@ from .registry import register
 
 @register("feed_forward", "dense")
 class DenseFeedForward(FeedForward):
+    takes_deferred_norm = True
+
     def __init__(self, params, tensors):
         super().__init__(params, tensors)
         self.width, self.inner, self.activation = params["width"], params["inner"], params["activation"]

@@ -33,6 +33,14 @@ class _KernelNorm(Norm):
             stream.pending = None
         return out
 
+    def deferred_possible(self, step, rows):
+        return step.dtype_is_bf16 and K.Normalized.possible(rows, self.width)
+
+    def deferred(self, stream, step):
+        if stream.pending is not None or not self.deferred_possible(step, stream.x.shape[0]):
+            return None
+        return K.Normalized(stream.x, self.weight, self.bias, self.eps, self.KIND)
+
 
 @register("norm", "layer_norm")
 class LayerNorm(_KernelNorm):

@@ -167,6 +167,46 @@ def test_skinny_gemm_at_decode_sizes(m, n, k, splits, columns, dtype):
         assert rel_err(out, gelu_tanh(want + bias.cpu().double())) < (2e-6 if dtype == "float32" else 6e-3)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 100, 136), (8, 6400, 1600), (16, 333, 1608), (9, 517, 64), (13, 4800, 2048),
+                                   (3, 48, 1024), (16, 96, 1032)])
+@pytest.mark.parametrize("kind,with_shift", [("layer_norm", True), ("rms_norm", False)])
+@pytest.mark.parametrize("columns", [0, 8, 16, 28])
+def test_skinny_gemm_normalises_its_rows_itself(m, n, k, kind, with_shift, columns):
+    """The product of rows of the float32 residual stream that the kernel normalises itself against
+    float64, and against the norm kernel followed by the plain product."""
+    gen = torch.Generator().manual_seed(m * n + k)
+    x = (torch.randn(m, k + 12, generator=gen) * 3.0 + 0.7).to(DEV)[:, :k]        # pitch unlike the width
+    gamma = (1.0 + 0.2 * torch.randn(k, generator=gen)).to(DEV)
+    beta = (0.3 * torch.randn(k, generator=gen)).to(DEV) if with_shift else None
+    w = (torch.randn(n, k, generator=gen) / math.sqrt(k)).to(torch.bfloat16).to(DEV)
+    bias = torch.randn(n, generator=gen).to(DEV)
+    eps = 1e-5
+    xd = x.cpu().double()
+    if kind == "layer_norm":
+        h = (xd - xd.mean(-1, keepdim=True)) / torch.sqrt(xd.var(-1, unbiased=False, keepdim=True) + eps)
+    else:
+        h = xd / torch.sqrt((xd ** 2).mean(-1, keepdim=True) + eps)
+    h = h * gamma.cpu().double() + (beta.cpu().double() if with_shift else 0.0)
+    want = gelu_tanh(h @ w.cpu().double().t() + bias.cpu().double())
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    operand = K.Normalized(x, gamma, beta, eps, kind)
+    assert operand.shape == (m, k) and K.Normalized.possible(m, k)
+    K.gemm(operand, w, K.epilogue_act(out, "gelu_tanh", bias), variant=columns)
+    assert rel_err(out, want) < 6e-3
+    normed = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
+    K.add_norm(x.contiguous(), normed, gamma, beta, eps, kind)
+    apart = torch.empty_like(out)
+    K.gemm(normed, w, K.epilogue_act(apart, "gelu_tanh", bias), impl="skinny", variant=columns)
+    assert rel_err(out, apart.double()) < 4e-3            # the statistics are summed in another order: a last bit of a row's values
+    parts = torch.full((2, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    if k >= 256:
+        K.gemm(operand, w, K.epilogue_f32(parts), splits=2, variant=columns)
+        assert rel_err(parts.sum(0), h @ w.cpu().double().t()) < 6e-3
+    with pytest.raises(K.KernelError, match="up to 16 rows"):
+        K.gemm(K.Normalized(torch.zeros(17, k, device=DEV), gamma, beta, eps, kind), w,
+               K.epilogue_store(torch.empty(17, n, dtype=torch.bfloat16, device=DEV)))
+
+
 @pytest.mark.parametrize("impl,m,n,k,splits", [("skinny", 5, 96, 1600, 4), ("skinny", 64, 50, 6400, 8),
                                                ("skinny", 20, 1600, 320, 2), ("tile", 150, 200, 1600, 3)])
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])

@@ -72,6 +72,25 @@ class Normalized:
         return rows <= cls.MAX_ROWS and width <= cls.MAX_WIDTH and width % 8 == 0
 
 
+# Argument types of the entry points a step calls hundreds of times: with them declared, ctypes
+# converts plain Python integers itself, which costs a fraction of wrapping each in a ctypes object.
+_P = ctypes.POINTER
+_SIGNATURES = {
+    "bt_embed": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int],
+    "bt_add_norm": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_int,
+                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int],
+    "bt_gemm_plain": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue)],
+    "bt_gemm_tile": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue), _c_int, _c_int],
+    "bt_gemm_skinny": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue), _c_int, _c_int,
+                       _P(NormOperand)],
+    "bt_gemm_library_bf16": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue)],
+    "bt_attention_plain": [_c_ptr, _c_int, _P(AttnArgs)],
+    "bt_attention_f32": [_c_ptr, _P(AttnArgs)],
+    "bt_attention_prefill_bf16": [_c_ptr, _P(AttnArgs)],
+    "bt_attention_decode_bf16": [_c_ptr, _P(AttnArgs)],
+    "bt_kv_copy": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _P(KvView), _c_int, _c_int],
+}
+
 _modules = {}
 _lock = threading.Lock()
 
@@ -89,6 +108,9 @@ def _module(name):
             except OSError as error:
                 raise RuntimeError(f"cannot load the kernel library {path}: {error}") from error
             lib.bt_last_error.restype = ctypes.c_char_p
+            for entry, types in _SIGNATURES.items():
+                if hasattr(lib, entry):
+                    getattr(lib, entry).argtypes = types
             _modules[name] = lib
         return lib
 
@@ -248,9 +270,9 @@ def epilogue_qkv(q_out, n_q, n_kv, kv_view, tok_seq, tok_pos, bias=None):
 def embed(ids, positions, table, position_table, out):
     """out[t] = table[ids[t]] (+ position_table[positions[t]]); out is the float32 stream."""
     lib = _module("core")
-    _check(lib, lib.bt_embed(_c_ptr(_stream()), DTYPE_CODES[table.dtype], _c_ptr(ids.data_ptr()),
-                             _c_ptr(_ptr(positions)), _c_ptr(table.data_ptr()), _c_ptr(_ptr(position_table)),
-                             _c_ptr(out.data_ptr()), _c_int(ids.numel()), _c_int(table.shape[1])))
+    _check(lib, lib.bt_embed(_stream(), DTYPE_CODES[table.dtype], ids.data_ptr(),
+                             _ptr(positions), table.data_ptr(), _ptr(position_table),
+                             out.data_ptr(), ids.numel(), table.shape[1]))
 
 
 def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None, rows=None,
@@ -270,10 +292,10 @@ def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None,
         write_back = False      # nothing is added: the stream already holds what would be written
     out_dtype = DTYPE_CODES[out.dtype] if out is not None else FLOAT32
     _check(lib, lib.bt_add_norm(
-        _c_ptr(_stream()), _c_int(out_dtype), _c_ptr(x.data_ptr()), _c_ptr(_ptr(delta)), _c_int(n_delta),
-        _c_i64(stride), _c_ptr(_ptr(bias)), _c_ptr(_ptr(gamma)), _c_ptr(_ptr(beta)), _c_float(eps),
-        _c_int(NORM_KINDS[kind]), _c_ptr(_ptr(out)), _c_ptr(_ptr(rows)), _c_int(n_rows), _c_int(width),
-        _c_int(1 if write_back else 0)))
+        _stream(), out_dtype, x.data_ptr(), _ptr(delta), n_delta,
+        stride, _ptr(bias), _ptr(gamma), _ptr(beta), eps,
+        NORM_KINDS[kind], _ptr(out), _ptr(rows), n_rows, width,
+        1 if write_back else 0))
 
 
 def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
@@ -281,9 +303,10 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
 
     impl: "auto" (skinny up to 64 rows; beyond that the tile kernel, or for bfloat16 the vendor's
     library where it is usable and has the epilogue; float32 operands that are not multiples of
-    four wide go to the plain kernel), or one of "plain", "tile", "skinny", "library" to force one.  variant picks one of the tile kernel's forms
-    (0: the fastest the operands allow, 1: any K, 2: lean, 3: direct to LDS) or, for the skinny
-    kernel, the output columns a work-group owns (8, 12, ... 32; 0: chosen for balance).
+    four wide go to the plain kernel), or one of "plain", "tile", "skinny", "library" to force one.
+    variant picks one of the tile kernel's forms (0: the fastest the operands allow, 1: any K,
+    2: lean, 3: direct to LDS) or, for the skinny kernel, the output columns a work-group owns
+    (8, 12, ... 32; 0: chosen for balance).  ``a`` may be a :class:`Normalized`.
     """
     m, k = a.shape
     n = w.shape[0]
@@ -293,9 +316,8 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
         operand = NormOperand(x=a.x.data_ptr(), ldx=a.x.stride(0), gamma=a.gamma.data_ptr(), beta=_ptr(a.beta),
                               eps=a.eps, kind=NORM_KINDS[a.kind])
         lib = _module("gemm_mfma")
-        _check(lib, lib.bt_gemm_skinny(_c_ptr(_stream()), _c_int(BFLOAT16), None, _c_i64(0), _c_ptr(w.data_ptr()),
-                                       _c_int(m), _c_int(n), _c_int(k), ctypes.byref(epilogue), _c_int(splits),
-                                       _c_int(variant), ctypes.byref(operand)))
+        _check(lib, lib.bt_gemm_skinny(_stream(), BFLOAT16, None, 0, w.data_ptr(), m, n, k, epilogue, splits,
+                                       variant, operand))
         return
     if w.shape[1] != k or a.stride(1) != 1 or not w.is_contiguous() or a.dtype != w.dtype:
         raise KernelError(f"gemm: operands [{m},{k}] {a.dtype} and [{n},{w.shape[1]}] {w.dtype} do not fit")
@@ -322,13 +344,12 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
                     print(f"[burn_transformers_amd] {refusal}; this shape runs on the package's tile kernel",
                           file=sys.stderr, flush=True)
                     impl = "tile"
-    args = (_c_ptr(a.data_ptr()), _c_i64(a.stride(0)), _c_ptr(w.data_ptr()), _c_int(m), _c_int(n), _c_int(k),
-            ctypes.byref(epilogue))
+    args = (a.data_ptr(), a.stride(0), w.data_ptr(), m, n, k, epilogue)
     if impl == "plain":
         if splits != 1:
             raise KernelError("gemm: the plain kernel does not split K")
         lib = _module("core")
-        _check(lib, lib.bt_gemm_plain(_c_ptr(_stream()), _c_int(dtype), *args))
+        _check(lib, lib.bt_gemm_plain(_stream(), dtype, *args))
         return
     if impl == "library":
         if dtype != BFLOAT16:
@@ -338,13 +359,13 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
             raise KernelError("gemm: the vendor's GEMM library is not available")
         if splits != 1:
             raise KernelError("gemm: the library product does not split K")
-        _check(lib, lib.bt_gemm_library_bf16(_c_ptr(_stream()), *args))
+        _check(lib, lib.bt_gemm_library_bf16(_stream(), *args))
         return
     lib = _module("gemm_mfma")
     if impl == "tile":
-        _check(lib, lib.bt_gemm_tile(_c_ptr(_stream()), _c_int(dtype), *args, _c_int(splits), _c_int(variant)))
+        _check(lib, lib.bt_gemm_tile(_stream(), dtype, *args, splits, variant))
     else:
-        _check(lib, lib.bt_gemm_skinny(_c_ptr(_stream()), _c_int(dtype), *args, _c_int(splits), _c_int(variant), None))
+        _check(lib, lib.bt_gemm_skinny(_stream(), dtype, *args, splits, variant, None))
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
@@ -367,28 +388,28 @@ def attention(args, dtype, decode, impl="auto"):
             impl = "tiled" if args.kv.head_dim <= 128 and args.ldq % 4 == 0 else "plain"
     if impl == "plain":
         lib = _module("core")
-        _check(lib, lib.bt_attention_plain(_c_ptr(_stream()), _c_int(code), ctypes.byref(args)))
+        _check(lib, lib.bt_attention_plain(_stream(), code, args))
         return
     if impl == "tiled":
         if code != FLOAT32:
             raise KernelError("attention: the tiled kernel takes float32 only")
         lib = _module("attention_f32")
-        _check(lib, lib.bt_attention_f32(_c_ptr(_stream()), ctypes.byref(args)))
+        _check(lib, lib.bt_attention_f32(_stream(), args))
         return
     if code != BFLOAT16:
         raise KernelError("attention: the MFMA kernels take bfloat16 only")
     lib = _module(f"attention_bf16_hd{args.kv.head_dim}")
     fn = lib.bt_attention_decode_bf16 if decode else lib.bt_attention_prefill_bf16
-    _check(lib, fn(_c_ptr(_stream()), ctypes.byref(args)))
+    _check(lib, fn(_stream(), args))
 
 
 def kv_copy(k_rows, v_rows, tok_seq, tok_pos, kv_view, to_cache):
     """Copies [tokens, kv_heads * head_dim] rows into the paged cache, or back out of it."""
     lib = _module("core")
-    _check(lib, lib.bt_kv_copy(_c_ptr(_stream()), _c_int(DTYPE_CODES[k_rows.dtype]), _c_ptr(k_rows.data_ptr()),
-                               _c_ptr(v_rows.data_ptr()), _c_i64(k_rows.stride(0)), _c_ptr(tok_seq.data_ptr()),
-                               _c_ptr(tok_pos.data_ptr()), ctypes.byref(kv_view), _c_int(k_rows.shape[0]),
-                               _c_int(1 if to_cache else 0)))
+    _check(lib, lib.bt_kv_copy(_stream(), DTYPE_CODES[k_rows.dtype], k_rows.data_ptr(),
+                               v_rows.data_ptr(), k_rows.stride(0), tok_seq.data_ptr(),
+                               tok_pos.data_ptr(), kv_view, k_rows.shape[0],
+                               1 if to_cache else 0))
 
 
 _sample_workspaces = {}

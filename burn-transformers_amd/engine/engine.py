@@ -15,9 +15,12 @@ the same behind prefill and decode, src/models/llama/model/decode.rs:630-684).  
 validated before anything changes, lengths advance only after the forward pass was launched
 without error (decode.rs:38-41).
 
-Steps in which every sequence brings one token are replayed from a HIP graph per batch size:
-such a step is hundreds of short kernels, and launching them one by one costs more than
-running them.
+Steps are replayed from HIP graphs where their shape repeats: a step is hundreds of kernels,
+and launching them one by one costs the host several microseconds each, more than the short
+kernels of a decode step take to run.  A graph belongs to a shape (tokens, sequences, wanted
+rows, most tokens of one sequence); what differs between steps of one shape (ids, positions,
+block tables, wanted rows) lives in device tables that are filled before each replay.  Decode
+shapes are captured when they come the second time, other shapes the third time.
 """
 
 import numpy as np
@@ -27,6 +30,7 @@ from ..cache.storage import Cache
 from .step import BufferPool, Step, StepLayout, StepPlan
 
 _PINNED_RING = 4
+_MAX_GRAPHS = 48           # graphs kept; the one that was used longest ago goes first
 
 
 class StepError(ValueError):
@@ -46,8 +50,8 @@ class Engine:
         self._meta = None                  # device int32 buffer of eager steps
         self._pinned = []                  # ring of (pinned int32 tensor, event)
         self._pinned_next = 0
-        self._graphs = {}                  # n_seqs -> dict(graph, meta, logits, generation)
-        self._seen_decode = set()
+        self._graphs = {}                  # shape -> dict(graph, meta, logits, generation), in order of last use
+        self._seen = {}                    # shape -> times it came without a graph
         self.steps_run = 0
         self.graph_replays = 0
 
@@ -123,13 +127,10 @@ class Engine:
         plan = StepPlan(checked["slots"], checked["starts"], checked["counts"], checked["ids"],
                         checked["wanted"], [self.cache.blocks(s) for s in checked["slots"]],
                         self.cache.max_blocks)
-        if not checked["wanted"]:
-            logits = self._run_eager(plan, want_logits=False)
-        elif plan.decode and self.use_graphs and plan.layout.rows == plan.n_seqs and \
-                checked["wanted"] == list(range(plan.n_seqs)):
-            logits = self._run_decode_graph(plan)
+        if self.use_graphs:
+            logits = self._run_from_graph(plan, readout=bool(checked["wanted"]))
         else:
-            logits = self._run_eager(plan)
+            logits = self._run_eager(plan, want_logits=bool(checked["wanted"]))
         for slot, length in checked["new_lengths"].items():
             ledger.commit(slot, length)
         self.steps_run += 1
@@ -160,23 +161,29 @@ class Engine:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return self.model.forward(step, self.cache)
 
-    def _run_decode_graph(self, plan):
-        key = plan.n_seqs
-        held = self._graphs.get(key)
+    def _run_from_graph(self, plan, readout):
+        key = (plan.layout.key(), plan.max_count, readout)
+        held = self._graphs.pop(key, None)
         if held is not None and held["generation"] != self.pool.generation:
             held = None                                   # a workspace moved: the graph is stale
-            del self._graphs[key]
         if held is None:
-            if key not in self._seen_decode:              # first time: run eagerly, which also sizes the workspaces
-                self._seen_decode.add(key)
-                return self._run_eager(plan)
-            held = self._capture(plan)
+            # the first times a shape comes it runs eagerly, which also sizes the workspaces
+            seen = self._seen.get(key, 0)
+            if seen < (1 if plan.decode else 2):
+                if len(self._seen) > 4096:
+                    self._seen.clear()
+                self._seen[key] = seen + 1
+                return self._run_eager(plan, want_logits=readout)
+            held = self._capture(plan, readout)
+            while len(self._graphs) >= _MAX_GRAPHS:
+                self._graphs.pop(next(iter(self._graphs)))
+        self._graphs[key] = held                          # (again) the most recently used
         self._upload(plan.host, held["meta"])
         held["graph"].replay()
         self.graph_replays += 1
         return held["logits"]
 
-    def _capture(self, plan):
+    def _capture(self, plan, readout):
         meta = torch.empty(plan.layout.total, dtype=torch.int32, device=self.device)
         self._upload(plan.host, meta)
         step = Step(plan.layout, meta, self.pool, self.dtype, plan)
@@ -185,9 +192,9 @@ class Engine:
         self.pool.frozen = True
         try:
             with torch.cuda.graph(graph):
-                logits = self.model.forward(step, self.cache)
+                logits = self.model.forward(step, self.cache, readout=readout)
         finally:
             self.pool.frozen = False
-        held = dict(graph=graph, meta=meta, logits=logits, generation=self.pool.generation)
-        self._graphs[plan.n_seqs] = held
-        return held
+        if not readout:
+            logits = torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        return dict(graph=graph, meta=meta, logits=logits, generation=self.pool.generation)

@@ -233,6 +233,43 @@ def test_graph_and_eager_decoding_agree_bitwise():
     assert torch.equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,chunk", [("A", 40), ("B", 70)])
+def test_prompt_steps_of_a_repeating_shape_are_replayed_from_graphs(name, dtype, chunk):
+    """Chunks of prompts whose shape repeats (same counts; other ids, positions, slots and wanted
+    places) run from a graph from the third time on, with the engine's eager steps and waits for the
+    device between the replays; every replay is bitwise what an engine without graphs computes."""
+    replayed = engine_for(name, dtype, max_tokens=64 * 8)
+    plain_engine = engine_for(name, dtype, max_tokens=64 * 8, graphs=False)
+    counts = [chunk, chunk - 9, 3]
+    replays_of_prompts = 0
+    for rep in range(4):
+        requests = prompts_for(name, [2 * c + 2 for c in counts], seed=50 + rep)
+        slots = [(replayed.open(), plain_engine.open()) for _ in requests]
+        if rep % 2:                         # other slots and blocks than last time
+            extra = (replayed.open(), plain_engine.open())
+        for part in range(2):               # two steps of the same shape, the second on a filled cache
+            want = [[(rep + part) % c, c - 1] for c in counts] if part else [[] for _ in counts]
+            entries = lambda which: [(s[which], r[part * c:(part + 1) * c]) for s, r, c in zip(slots, requests, counts)]
+            before = replayed.graph_replays
+            got = replayed.step(entries(0), want).clone()
+            replays_of_prompts += replayed.graph_replays - before
+            torch.cuda.synchronize()
+            assert torch.equal(got, plain_engine.step(entries(1), want)), (rep, part)
+        for t in range(2):                  # single tokens in between: graphs of their own
+            entries = lambda which: [(s[which], [r[2 * c + t]]) for s, r, c in zip(slots, requests, counts)]
+            assert torch.equal(replayed.step(entries(0)).clone(), plain_engine.step(entries(1)))
+        if rep == 3:
+            rows = [2 * c - 1 for c in counts]
+            for (slot, _), request, row in zip(slots, requests, rows):
+                assert replayed.length(slot) == len(request)
+        for pair in slots + ([extra] if rep % 2 else []):
+            replayed.close(pair[0])
+            plain_engine.close(pair[1])
+    assert replays_of_prompts >= 3          # each kind of step came four times: twice eagerly, then captured and replayed
+    replayed.cache.ledger.check()
+
+
 def test_refused_steps_change_nothing():
     engine = engine_for("A", "float32", max_tokens=128)
     slot = engine.open()

@@ -22,6 +22,8 @@ from .registry import register
 
 @register("mixer", "attention")
 class CausalSelfAttention(Mixer):
+    takes_deferred_norm = True
+
     def __init__(self, params, tensors):
         super().__init__(params, tensors)
         p = params

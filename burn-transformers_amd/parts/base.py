@@ -110,6 +110,9 @@ class Norm(Part):
 
 
 class Mixer(Part):
+    # True for a mixer that hands ``h`` to ``kernels.library.gemm`` and looks at nothing but its
+    # shape (see FeedForward.takes_deferred_norm)
+    takes_deferred_norm = False
     # False for a mixer whose forward reads the step's host tables (``step.host``) or otherwise
     # does per-step work in Python: steps of a model with such a mixer are never graph-replayed
     graph_safe = True

@@ -270,6 +270,48 @@ def test_prompt_steps_of_a_repeating_shape_are_replayed_from_graphs(name, dtype,
     replayed.cache.ledger.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_random_schedule_with_and_without_graphs(dtype):
+    """A hundred steps of random shape from a small set (so that shapes repeat and are replayed from
+    graphs), sequences that end and slots that are used again: the engine with graphs and the one
+    without give the same bits at every step, and the last logits of every sequence are the plain
+    implementation's."""
+    import random
+    name = "B"
+    limit = CONFIGS[name][0]["n_positions"]
+    replayed = engine_for(name, dtype, max_tokens=64 * 12)
+    eager = engine_for(name, dtype, max_tokens=64 * 12, graphs=False)
+    rng = random.Random(7)
+    live = {}                                   # request number -> dict(slots, tokens, fed)
+    next_request = 0
+    for step_number in range(100):
+        while len(live) < 4 and (len(live) < 2 or rng.random() < 0.3):
+            tokens = prompts_for(name, [rng.choice([30, 64, 100, 150])], seed=100 + next_request)[0]
+            live[next_request] = dict(slots=(replayed.open(), eager.open()), tokens=tokens, fed=0)
+            next_request += 1
+        chosen = [r for r in live if rng.random() < 0.9] or list(live)
+        width = rng.choice([1, 1, 1, 7, 33])            # most steps bring one token per sequence
+        counts = {r: min(width if rng.random() < 0.9 else 2, len(live[r]["tokens"]) - live[r]["fed"]) for r in chosen}
+        entries = lambda which: [(live[r]["slots"][which], live[r]["tokens"][live[r]["fed"]:live[r]["fed"] + counts[r]])
+                                 for r in chosen]
+        want = [[counts[r] - 1] if rng.random() < 0.8 else [] for r in chosen]
+        got = replayed.step(entries(0), want).clone()
+        assert torch.equal(got, eager.step(entries(1), want)), f"step {step_number}"
+        row = 0
+        for r, places in zip(chosen, want):
+            live[r]["fed"] += counts[r]
+            if places:
+                if live[r]["fed"] == len(live[r]["tokens"]):
+                    check(got[row:row + 1], plain_logits(name, live[r]["tokens"])[-1:], dtype, f"request {r}")
+                row += 1
+            if live[r]["fed"] == len(live[r]["tokens"]):
+                replayed.close(live[r]["slots"][0])
+                eager.close(live[r]["slots"][1])
+                del live[r]
+        replayed.cache.ledger.check()
+    assert replayed.graph_replays > 10, replayed.graph_replays
+
+
 def test_refused_steps_change_nothing():
     engine = engine_for("A", "float32", max_tokens=128)
     slot = engine.open()

@@ -17,8 +17,8 @@
 //     cache's value layout (four positions interleaved per channel) makes a lane's read of four
 //     keys one 16-byte LDS read, against the probabilities (broadcast reads).
 // A query's result depends on its own keys and on the block boundaries only, which lie at
-// multiples of 64 positions whatever the step: the same arithmetic in the same order whether the
-// query comes alone (decoding) or inside a prompt.
+// multiples of 64 positions whatever the step: the same arithmetic in the same order whatever
+// else the step holds.  (Steps of one token per sequence have a kernel of their own, below.)
 //
 // Head sizes: multiples of 16 up to 128.
 
@@ -200,6 +200,117 @@ attention_f32_kernel(AttnArgs a) {
   }
 }
 
+// One token per sequence (a decode step): the tiled kernel above would give each work-group a
+// single query and leave three of its four waves only the staging.  Here a work-group still
+// takes one (sequence, head), but its four waves take the blocks of 64 keys in turn and read them
+// straight from the cache: scores with lane = key (a lane reads its own key's row, the query comes
+// from LDS as a broadcast), the block's softmax statistics as wave reductions, values with lane =
+// channel (four keys per 16-byte read, as the cache lays them out; the probabilities come back
+// from LDS as broadcasts).  The four waves' running results meet in LDS at the end.
+template <int CPT>
+__global__ void __launch_bounds__(256)
+attention_f32_decode_kernel(AttnArgs a) {
+  constexpr int MAX_HD = 64 * CPT;
+  __shared__ __attribute__((aligned(16))) float qs[MAX_HD];
+  __shared__ __attribute__((aligned(16))) float ps[4][BT_KV_BLOCK];
+  __shared__ float part_max[4], part_sum[4];
+  __shared__ __attribute__((aligned(16))) float part_acc[4][MAX_HD];
+  const int hd = a.kv.head_dim;
+  const int seq = blockIdx.x, head = blockIdx.y, kv_head = head / (a.q_heads / a.kv.kv_heads);
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pos = a.seq_start[seq];                     // the query's position: token `seq` of the step
+  const float* q = static_cast<const float*>(a.q) + (int64_t)seq * a.ldq + head * hd;
+  if (tid < hd) qs[tid] = q[tid];
+  __syncthreads();
+  const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  const int first_block = lo / BT_KV_BLOCK, last_block = pos / BT_KV_BLOCK;
+  const float* keys = static_cast<const float*>(a.kv.keys);
+  const float* values = static_cast<const float*>(a.kv.values);
+  float run_max = -INFINITY, run_sum = 0.f, acc[CPT];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) acc[j] = 0.f;
+  for (int block = first_block + wave; block <= last_block; block += 4) {
+    int physical = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + block];
+    int64_t base = ((int64_t)physical * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * hd);
+    // this lane's key: row `lane` of the block
+    const float4* krow = reinterpret_cast<const float4*>(keys + base + (int64_t)lane * hd);
+    const int quads = hd >> 2;
+    float4 kreg[16 * CPT];                     // the whole row in flight at once: one trip to memory, not sixteen
+#pragma unroll
+    for (int c4 = 0; c4 < 16 * CPT; ++c4) kreg[c4] = krow[c4 < quads ? c4 : 0];
+    float s = 0.f;
+#pragma unroll
+    for (int c4 = 0; c4 < 16 * CPT; ++c4) {
+      if (c4 < quads) {
+        float4 q4 = *reinterpret_cast<const float4*>(qs + c4 * 4);
+        s = fmaf(q4.x, kreg[c4].x, s);
+        s = fmaf(q4.y, kreg[c4].y, s);
+        s = fmaf(q4.z, kreg[c4].z, s);
+        s = fmaf(q4.w, kreg[c4].w, s);
+      }
+    }
+    const int key_pos = block * BT_KV_BLOCK + lane;
+    const bool seen = key_pos <= pos && key_pos >= lo;
+    const float score = seen ? s * a.scale : -INFINITY;
+    const float new_max = fmaxf(run_max, wave_max(score));          // finite: the block holds at least one seen key
+    const float p = expf(score - new_max);
+    const float rescale = expf(run_max - new_max);                  // exp(-inf) = 0 at the wave's first block
+    run_sum = fmaf(run_sum, rescale, wave_sum(p));
+    run_max = new_max;
+    ps[wave][lane] = p;                                             // read back below by this wave only
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) acc[j] *= rescale;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int channel = lane + 64 * j;
+      const int cc = channel < hd ? channel : 0;
+      float4 vreg[BT_KV_BLOCK / 4];            // the channel's 64 values in flight at once
+#pragma unroll
+      for (int k4 = 0; k4 < BT_KV_BLOCK / 4; ++k4)
+        vreg[k4] = *reinterpret_cast<const float4*>(values + base + (int64_t)(k4 * hd + cc) * 4);
+#pragma unroll
+      for (int k4 = 0; k4 < BT_KV_BLOCK / 4; ++k4) {
+        float4 p4 = *reinterpret_cast<const float4*>(&ps[wave][k4 * 4]);
+        // a position that holds no token yet may hold anything (0 * NaN is NaN): not multiplied
+        acc[j] = p4.x != 0.f ? fmaf(p4.x, vreg[k4].x, acc[j]) : acc[j];
+        acc[j] = p4.y != 0.f ? fmaf(p4.y, vreg[k4].y, acc[j]) : acc[j];
+        acc[j] = p4.z != 0.f ? fmaf(p4.z, vreg[k4].z, acc[j]) : acc[j];
+        acc[j] = p4.w != 0.f ? fmaf(p4.w, vreg[k4].w, acc[j]) : acc[j];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");          // the probabilities are overwritten next turn
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) {
+    part_max[wave] = run_max;
+    part_sum[wave] = run_sum;
+  }
+#pragma unroll
+  for (int j = 0; j < CPT; ++j)
+    if (lane + 64 * j < hd) part_acc[wave][lane + 64 * j] = acc[j];
+  __syncthreads();
+  if (wave == 0) {
+    float top = fmaxf(fmaxf(part_max[0], part_max[1]), fmaxf(part_max[2], part_max[3]));
+    float* out = static_cast<float*>(a.out) + (int64_t)seq * a.ldo + head * hd;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      int channel = lane + 64 * j;
+      if (channel >= hd) continue;
+      float num = 0.f, den = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {                                 // a wave that had no block: maximum -inf, weight 0
+        float f = part_max[w] == -INFINITY ? 0.f : expf(part_max[w] - top);
+        num = fmaf(part_acc[w][channel], f, num);
+        den = fmaf(part_sum[w], f, den);
+      }
+      out[channel] = den > 0.f ? num / den : 0.f;
+    }
+  }
+}
+
 BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
   const AttnArgs& a = *args;
   if (a.n_tokens <= 0 || a.n_seqs <= 0) return BT_OK;
@@ -214,6 +325,14 @@ BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
     BT_REFUSE("attention_f32: missing operand");
   if (a.ldq % 4 != 0 || ((uintptr_t)a.q & 15) || ((uintptr_t)a.kv.keys & 15) || ((uintptr_t)a.kv.values & 15))
     BT_REFUSE("attention_f32: queries, keys and values are read 16 bytes at a time (row pitch %lld)", (long long)a.ldq);
+  if (a.max_count == 1 && a.n_tokens == a.n_seqs) {      // a decode step: one token per sequence, in their order
+    dim3 grid(a.n_seqs, a.q_heads);
+    if (hd <= 64)
+      hipLaunchKernelGGL(attention_f32_decode_kernel<1>, grid, dim3(256), 0, (hipStream_t)stream, a);
+    else
+      hipLaunchKernelGGL(attention_f32_decode_kernel<2>, grid, dim3(256), 0, (hipStream_t)stream, a);
+    return bt_check_launch("attention_f32");
+  }
   const int q_tiles = (a.max_count + F32_QUERIES - 1) / F32_QUERIES;
   dim3 grid(a.n_seqs * q_tiles, a.q_heads), block(256);
   auto lds_bytes = [](int max_hd) {

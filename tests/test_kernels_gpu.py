@@ -327,7 +327,7 @@ def test_attention_tiled_float32(q_heads, kv_heads, hd, totals, counts, window):
     K.attention(args, dt, decode=max(counts) == 1, impl="tiled")
     want = case.reference(q, q_heads, scale, window)
     assert rel_err(out, want) < 3e-6
-    # the last token of every sequence alone, as a decode step would bring it
+    # the last token of every sequence alone, as a decode step brings it (a kernel of its own)
     last = [int(case.seq_off[i + 1]) - 1 for i in range(len(totals))]
     alone = PagedCase(totals, [1] * len(totals), kv_heads, hd, dt, DEV, seed=2, poison=True)
     q1 = q[last].contiguous()
@@ -335,7 +335,24 @@ def test_attention_tiled_float32(q_heads, kv_heads, hd, totals, counts, window):
     args = K.attention_args(q1, out1, alone.view(), alone.tok_seq, alone.tok_pos, alone.seq_off, alone.seq_start,
                             q_heads, len(totals), 1, scale, window)
     K.attention(args, dt, decode=True, impl="tiled")
-    assert torch.equal(out1, out[last])
+    assert rel_err(out1, want[last]) < 3e-6
+    # the last two tokens of every sequence that has two: the tiled kernel again, and bitwise what
+    # it gave the same queries among the others of their step
+    pairs = [i for i, c in enumerate(counts) if c >= 2]
+    if pairs:
+        sub_totals = [totals[i] for i in pairs]
+        two = PagedCase(totals, [2 if i in pairs else 1 for i in range(len(totals))], kv_heads, hd, dt, DEV, seed=2,
+                        poison=True)
+        rows = []
+        for i in range(len(totals)):
+            rows += [last[i] - 1, last[i]] if i in pairs else [last[i]]
+        q2 = q[rows].contiguous()
+        out2 = torch.full((len(rows), q_heads * hd), float("nan"), dtype=dt, device=DEV)
+        args = K.attention_args(q2, out2, two.view(), two.tok_seq, two.tok_pos, two.seq_off, two.seq_start,
+                                q_heads, len(totals), 2, scale, window)
+        K.attention(args, dt, decode=False, impl="tiled")
+        keep = [r for r, row in enumerate(rows) if (row in last and any(row == last[i] for i in pairs)) or row + 1 in last]
+        assert torch.equal(out2[keep], out[[rows[r] for r in keep]])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -82,6 +82,23 @@ class CacheLedger:
     def live(self, slot):
         return self.slots.held(slot)
 
+    def live_slots(self):
+        return [slot for slot in range(self.slots.count) if self.slots.held(slot)]
+
+    def truncate(self, slot, length):
+        """Rewinds a live sequence to ``length`` tokens: the blocks it no longer needs go back
+        (src/models/llama/model/decode.rs:386-395 rewinds a row the same way; to zero it empties it)."""
+        if not self.slots.held(slot):
+            raise ValueError(f"slot {slot} is not live")
+        if not (0 <= length <= self.lengths[slot]):
+            raise ValueError(f"slot {slot} holds {self.lengths[slot]} tokens and cannot be rewound to {length}")
+        keep = self.blocks_for(length)
+        for group in range(self.n_groups):
+            held = self.held_blocks[group][slot]
+            while len(held) > keep:
+                self.blocks[group].give(held.pop())
+        self.lengths[slot] = length
+
     # --- growth ----------------------------------------------------------------------------
     @staticmethod
     def blocks_for(length):

@@ -108,6 +108,13 @@ class Cache:
     def release(self, slot):
         self.ledger.release(slot)
 
+    def truncate(self, slot, length):
+        """Rewinds a sequence; refused where a mixer keeps state of fixed size, which only ever
+        holds the state after the last token (src/cache/tensor/recurrent.rs:3-8)."""
+        if self.state_groups and length != self.ledger.lengths[slot]:
+            raise ValueError("a model with fixed-size state per sequence cannot be rewound")
+        self.ledger.truncate(slot, length)
+
     def length(self, slot):
         return self.ledger.lengths[slot]
 

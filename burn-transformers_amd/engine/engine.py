@@ -67,6 +67,15 @@ class Engine:
     def length(self, slot):
         return self.cache.length(slot)
 
+    def truncate(self, slot, length):
+        """Rewinds a sequence to its first ``length`` tokens; later steps go on from there."""
+        self.cache.truncate(slot, length)
+
+    def reset(self):
+        """Ends every sequence (the reference's reset, src/architecture/traits.rs:64)."""
+        for slot in self.cache.ledger.live_slots():
+            self.cache.release(slot)
+
     # --- the step function -----------------------------------------------------------------
     def plan(self, entries, want=None):
         """Validates a step and lays its tables out on the host.  Changes nothing."""

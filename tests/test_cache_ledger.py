@@ -93,3 +93,28 @@ def test_random_traffic_keeps_the_invariants():
         ledger.release(slot)
     ledger.check()
     assert ledger.blocks[0].available() == 40 and ledger.slots.available() == 12
+
+
+def test_truncate_gives_blocks_back_and_keeps_the_rest():
+    ledger = CacheLedger(1, 8, 4, 8)
+    a, b = ledger.acquire(), ledger.acquire()
+    for slot, length in ((a, 200), (b, 70)):
+        ledger.check_growth({slot: length})
+        ledger.reserve(slot, length)
+        ledger.commit(slot, length)
+    assert ledger.blocks[0].available() == 8 - 4 - 2
+    kept = list(ledger.held_blocks[0][a][:2])
+    ledger.truncate(a, 65)                      # 65 tokens need two of the four blocks
+    assert ledger.lengths[a] == 65 and ledger.held_blocks[0][a] == kept
+    assert ledger.blocks[0].available() == 8 - 2 - 2
+    ledger.check()
+    ledger.truncate(a, 0)                       # to zero: the slot stays live and holds nothing
+    assert ledger.live(a) and ledger.held_blocks[0][a] == [] and ledger.live_slots() == [a, b]
+    with pytest.raises(ValueError, match="cannot be rewound to 71"):
+        ledger.truncate(b, 71)
+    with pytest.raises(ValueError, match="not live"):
+        ledger.truncate(3, 0)
+    ledger.check_growth({a: 130})
+    ledger.reserve(a, 130)
+    ledger.commit(a, 130)
+    ledger.check()

@@ -312,6 +312,34 @@ def test_random_schedule_with_and_without_graphs(dtype):
     assert replayed.graph_replays > 10, replayed.graph_replays
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rewound_sequences_go_on_as_if_the_rest_had_never_been(dtype):
+    """truncate() rewinds a sequence (the blocks it no longer needs go back), other tokens are fed
+    from there, and the logits are those of the new sequence; reset() ends everything."""
+    name = "B"
+    engine = engine_for(name, dtype, max_tokens=64 * 6)
+    first, second = prompts_for(name, [150, 100], seed=61)
+    a, b = engine.open(), engine.open()
+    engine.step([(a, first), (b, second)])
+    free_before = engine.cache.ledger.blocks[0].available()
+    engine.truncate(a, 70)                                  # 150 -> 70 tokens: one of three blocks goes back
+    assert engine.length(a) == 70 and engine.cache.ledger.blocks[0].available() == free_before + 1
+    other = prompts_for(name, [40], seed=62)[0]
+    logits = engine.step([(a, other), (b, [5])], want=[list(range(40)), [0]])
+    check(logits[:40], plain_logits(name, first[:70] + other)[70:], dtype, "after the rewind")
+    check(logits[40:], plain_logits(name, second + [5])[-1:], dtype, "the other sequence")
+    engine.truncate(a, 0)                                   # to nothing: the slot stays open
+    logits = engine.step([(a, other[:9])], want=[[8]])
+    check(logits, plain_logits(name, other[:9])[-1:], dtype, "from the start again")
+    with pytest.raises(ValueError, match="cannot be rewound"):
+        engine.truncate(a, 10)
+    engine.cache.ledger.check()
+    engine.reset()
+    assert engine.cache.ledger.live_slots() == [] and \
+        engine.cache.ledger.blocks[0].available() == engine.cache.ledger.blocks[0].count
+    engine.cache.ledger.check()
+
+
 def test_refused_steps_change_nothing():
     engine = engine_for("A", "float32", max_tokens=128)
     slot = engine.open()

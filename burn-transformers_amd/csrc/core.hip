@@ -701,6 +701,10 @@ sample_select_kernel(const float* __restrict__ logits, int64_t ld, int vocab, in
   for (int c = 0; c < chunks; ++c)
     if (part[c].top > top) { top = part[c].top; arg = part[c].arg; }   // chunks in index order: `>` keeps the lowest
   auto scaled = [&](int c) { return part[c].top == -INFINITY ? 0.f : part[c].sum * expf(part[c].top - top); };
+  if (top == -INFINITY) {            // every score is -inf (all tokens excluded): nothing can be chosen
+    if (tid == 0) { ids[row] = 0; logp[row] = -INFINITY; }
+    return;
+  }
   float total = 0.f;
   for (int c = 0; c < chunks; ++c) total += scaled(c);                  // in index order
   if (!sample) {
@@ -1036,6 +1040,53 @@ select_processed_kernel(ProcessArgs a) {
     a.logp[row] = logf(shared_f[0]) - logf(total);
   }
   (void)shared_i;
+}
+
+// Steps 1 to 5 alone, element by element, into `out`: many work-groups per row, because one
+// compute unit pulls a row of logits and its two rows of counts (600 KB at a vocabulary of 50,257)
+// no faster than in 25 us.  What follows then reads processed scores only: plain greedy selection
+// or sampling (bt_sample, with temperature 1: it is already applied), or the truncating kernel
+// above with its own processing switched off.
+#define PROCESS_CHUNK 2048
+__global__ void __launch_bounds__(256)
+process_scores_kernel(ProcessArgs a, float* __restrict__ out, int64_t ldo) {
+  const int row = blockIdx.y, lo = blockIdx.x * PROCESS_CHUNK;
+  const int hi = lo + PROCESS_CHUNK < a.vocab ? lo + PROCESS_CHUNK : a.vocab;
+  const int brow = a.batch_rows ? a.batch_rows[row] : row;
+  const float* zrow = a.logits + (int64_t)row * a.ld;
+  float* orow = out + (int64_t)row * ldo;
+  for (int k = lo + threadIdx.x; k < hi; k += 256) {
+    float v = zrow[k];
+    if (a.bias != nullptr) v += a.bias[k];
+    if (a.counts_all != nullptr && a.repetition != 1.0f && a.counts_all[(int64_t)brow * a.counts_ld + k] > 0)
+      v = v < 0.f ? v * a.repetition : v / a.repetition;
+    if (a.counts_add != nullptr) {
+      const int c = a.counts_add[(int64_t)brow * a.counts_ld + k];
+      if (a.frequency != 0.f) v -= fminf(fmaxf(a.frequency * (float)c, -FLT_MAX), FLT_MAX);
+      if (a.presence != 0.f && c > 0) v -= a.presence;
+    }
+    if (a.sample) v /= a.temperature;
+    if (a.clamp) v = fminf(v, FLT_MAX);
+    orow[k] = v;
+  }
+  if (a.ban_ids == nullptr) return;
+  __syncthreads();                         // this work-group's own scores are written: now its banned ones
+  for (int j = a.ban_offsets[row] + threadIdx.x; j < a.ban_offsets[row + 1]; j += 256) {
+    const int k = a.ban_ids[j];
+    if (k >= lo && k < hi) orow[k] = -INFINITY;
+  }
+}
+
+BT_EXPORT int bt_process_scores(void* stream, const ProcessArgs* args, int rows, float* out, int64_t ldo) {
+  if (rows <= 0) return BT_OK;
+  const ProcessArgs& a = *args;
+  if (a.vocab <= 0 || a.logits == nullptr || out == nullptr || ldo < a.vocab) BT_REFUSE("process_scores: missing operand");
+  if (a.sample && !(a.temperature > 0.f)) BT_REFUSE("process_scores: temperature %g must be positive", (double)a.temperature);
+  if (!(a.repetition > 0.f)) BT_REFUSE("process_scores: repetition penalty %g must be positive", (double)a.repetition);
+  if ((a.ban_ids == nullptr) != (a.ban_offsets == nullptr)) BT_REFUSE("process_scores: banned tokens need their offsets");
+  dim3 grid((a.vocab + PROCESS_CHUNK - 1) / PROCESS_CHUNK, rows);
+  hipLaunchKernelGGL(process_scores_kernel, grid, dim3(256), 0, (hipStream_t)stream, a, out, ldo);
+  return bt_check_launch("process_scores");
 }
 
 BT_EXPORT int bt_select_processed(void* stream, const ProcessArgs* args, int rows) {

@@ -454,16 +454,35 @@ def select_processed(logits, ids, logp, *, bias=None, counts_all=None, counts_ad
     lib = _module("core")
     rows, vocab = logits.shape
     counts = counts_all if counts_all is not None else counts_add
+    sampling = temperature is not None
+    truncating = sampling and ((top_k or 0) > 0 or (top_p is not None and top_p < 1.0) or (min_p or 0.0) > 0.0)
     args = ProcessArgs(
         logits=logits.data_ptr(), ld=logits.stride(0), vocab=vocab, bias=_ptr(bias),
         counts_all=_ptr(counts_all), counts_add=_ptr(counts_add), counts_ld=counts.stride(0) if counts is not None else 0,
         batch_rows=_ptr(batch_rows), ban_ids=_ptr(ban_ids), ban_offsets=_ptr(ban_offsets),
         repetition=repetition, presence=presence, frequency=frequency,
-        sample=1 if temperature is not None else 0, temperature=temperature if temperature is not None else 1.0,
+        sample=1 if sampling else 0, temperature=temperature if sampling else 1.0,
         clamp=1 if clamp else 0, top_k=top_k or 0, top_p=top_p if top_p is not None else 1.0,
         min_p=min_p or 0.0, seed=seed & (2 ** 64 - 1), first_draw=first_draw & (2 ** 64 - 1),
         ids=ids.data_ptr(), logp=logp.data_ptr())
-    _check(lib, lib.bt_select_processed(_c_ptr(_stream()), ctypes.byref(args), _c_int(rows)))
+    if truncating:          # one work-group holds the row in registers: processing, thresholds and the draw in one kernel
+        _check(lib, lib.bt_select_processed(_c_ptr(_stream()), ctypes.byref(args), _c_int(rows)))
+        return
+    # Nothing is cut off: the processing alone by many work-groups per row into processed scores
+    # (one compute unit pulls a row's logits and counts no faster than in 25 us), then the plain
+    # selection: the lowest index of the maximum, or a draw at temperature 1 (it is applied already).
+    held = _processed_scores.get(logits.device)
+    if held is None or held.shape[0] < rows or held.shape[1] != vocab:
+        held = torch.empty((max(rows, 8), vocab), dtype=torch.float32, device=logits.device)
+        _processed_scores[logits.device] = held
+    scores = held[:rows]
+    _check(lib, lib.bt_process_scores(_c_ptr(_stream()), ctypes.byref(args), _c_int(rows),
+                                      _c_ptr(scores.data_ptr()), _c_i64(scores.stride(0))))
+    sample(scores, ids, logp, temperature=1.0 if sampling else None, seed=seed, first_draw=first_draw,
+           draw_rows=batch_rows)
+
+
+_processed_scores = {}
 
 
 def count_tokens(counts, rows, tokens):

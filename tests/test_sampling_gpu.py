@@ -34,7 +34,7 @@ def run_kernel(logits, batch_rows, **kw):
     return ids.tolist(), logp.tolist()
 
 
-@pytest.mark.parametrize("vocab", [517, 50257])
+@pytest.mark.parametrize("vocab", [517, 50257, 70001])
 def test_greedy_after_bias_penalties_and_bans(vocab):
     rows = 6
     logits, counts_all, counts_gen = make_rows(rows, vocab, seed=vocab)
@@ -95,6 +95,15 @@ def test_sampling_from_the_truncated_distribution(vocab, case):
             lo = float(c[k - 1]) if k > 0 else 0.0
             assert lo - 1e-4 <= u <= float(c[k]) + 1e-4, (r, k, u)
     assert checked >= rows - 2
+
+
+def test_cutting_off_is_refused_beyond_what_a_work_group_holds():
+    logits = torch.zeros(2, 70001)
+    with pytest.raises(K.KernelError, match="outside 1..65536"):
+        run_kernel(logits, [0, 1], temperature=1.0, top_k=5)
+    ids, logp = run_kernel(logits, [0, 1], temperature=1.0, repetition=1.3,
+                           counts_all=torch.ones(2, 70001, dtype=torch.int32))      # nothing cut off: any size
+    assert all(0 <= i < 70001 for i in ids)
 
 
 def test_rows_where_everything_is_tied_or_banned():

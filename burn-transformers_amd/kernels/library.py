@@ -72,8 +72,9 @@ class Normalized:
         return rows <= cls.MAX_ROWS and width <= cls.MAX_WIDTH and width % 8 == 0
 
 
-# Argument types of the entry points a step calls hundreds of times: with them declared, ctypes
-# converts plain Python integers itself, which costs a fraction of wrapping each in a ctypes object.
+# Argument types of the entry points a step calls hundreds of times: with them declared, plain
+# Python integers, None and structures can be passed as they are, and a wrong count of arguments
+# is an error at the call instead of garbage in a register.
 _P = ctypes.POINTER
 _SIGNATURES = {
     "bt_embed": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int],

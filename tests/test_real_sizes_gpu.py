@@ -1,4 +1,7 @@
-"""The engine at the layer sizes of GPT-2 XL (width 1600, 25 heads of 64, inner 6400, vocabulary
+"""The engine at the sizes of real models: two layers of GPT-2 XL's width, and all twelve layers
+of GPT-2 small's (at the end of the file).
+
+The engine at the layer sizes of GPT-2 XL (width 1600, 25 heads of 64, inner 6400, vocabulary
 50257, 1,024 positions) with two layers, against the plain implementation in float64: the sizes
 the measured kernels run at (columns per work-group chosen by balance, split K, paired and
 LDS-shared prefill attention, hundreds of keys per query) are not the tiny configurations'.
@@ -138,3 +141,47 @@ def test_unequal_batches_one_after_another(dtype):
             check(torch.cat(got[i]), plain_rows(r, rows[i]), dtype, f"batch {b} request {i}")
         engine.cache.ledger.check()
     assert set(seen[0]) & set(seen[1]), "slots were not used again"
+
+
+# --- GPT-2 small's sizes with all twelve layers, in float32 and in bfloat16: depth ----------------
+
+SMALL = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 12, "n_embd": 768, "n_head": 12,
+         "n_inner": 3072, "vocab_size": 50257, "n_positions": 1024, "activation_function": "gelu_new",
+         "layer_norm_epsilon": 1e-5, "scale_attn_by_inverse_layer_idx": False}
+_small = {}
+
+
+def small_model():
+    if not _small:
+        holder = tempfile.TemporaryDirectory(prefix="bt_small_")
+        weights = bt.write_random_model(holder.name, SMALL, 4)
+        _small.update(holder=holder, weights={k: (v.to(torch.bfloat16).float() if v.dim() == 2 else v.float())
+                                              for k, v in weights.items()}, models={})
+    return _small["holder"].name, _small["weights"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_twelve_layers_of_gpt2_small(dtype):
+    """A ragged batch of three prompts in one step, then eight tokens each one by one, through all
+    twelve layers of GPT-2 small's sizes: what an error that grows with depth would show."""
+    folder, weights = small_model()
+    if dtype not in _small["models"]:
+        _small["models"][dtype] = bt.load_model(folder, dtype=dtype, device="cuda:0")
+    engine = bt.Engine(_small["models"][dtype], max_tokens=2048)
+    gen = torch.Generator().manual_seed(9)
+    lengths = [1000, 301, 17]
+    requests = [torch.randint(0, SMALL["vocab_size"], (n + 8,), generator=gen).tolist() for n in lengths]
+    slots = [engine.open() for _ in requests]
+    wants = [[0, n // 2, n - 1] for n in lengths]
+    rows = [list(w) for w in wants]
+    logits = engine.step([(s, r[:n]) for s, r, n in zip(slots, requests, lengths)], want=wants).clone()
+    got = [[logits[3 * i:3 * i + 3]] for i in range(3)]
+    for t in range(8):
+        logits = engine.step([(s, [r[n + t]]) for s, r, n in zip(slots, requests, lengths)]).clone()
+        for i, n in enumerate(lengths):
+            got[i].append(logits[i:i + 1])
+            rows[i].append(n + t)
+    for i, request in enumerate(requests):
+        check(torch.cat(got[i]), plain.forward(request, weights, SMALL, rows=rows[i]), dtype, f"request {i}")
+    for slot in slots:
+        engine.close(slot)

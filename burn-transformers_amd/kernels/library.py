@@ -133,7 +133,8 @@ class one_stream:
     """While this context is open every kernel goes to the stream that was current when it was
     entered, looked up once: asking torch for the current stream costs more host time than a launch
     does, and a step is hundreds of launches.  Enter it inside whatever chose the stream (a
-    ``torch.cuda.stream`` or ``torch.cuda.graph`` context), never around it."""
+    ``torch.cuda.stream`` or ``torch.cuda.graph`` context), never around it.  One thread issues
+    kernels at a time (the same holds for the workspaces this module keeps per device)."""
 
     def __enter__(self):
         self.before = _held_stream[0]

@@ -23,6 +23,7 @@ class CausalLM:
     def __init__(self, plan, store, config=None, family=None):
         self.plan, self.store, self.config, self.family = plan, store, config, family
         self.dtype, self.device = store.dtype, store.device
+        self.load_report = getattr(store, "report", None)      # what loading did with the checkpoint's tensors
         self.width, self.vocab_size, self.max_positions = plan.width, plan.vocab_size, plan.max_positions
         self.embedding = build_part("embedding", plan.embedding, store)
         self.blocks = []

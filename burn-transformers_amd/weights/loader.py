@@ -27,11 +27,17 @@ def compute_dtype(name):
 
 
 class WeightStore(dict):
-    """name -> tensor on the device, in the layout the parts use; remembers how to undo it."""
+    """name -> tensor on the device, in the layout the parts use; remembers how to undo it, and
+    what loading did (``report``: the reference's LoadReport, src/checkpoint/report.rs)."""
 
     def __init__(self, dtype, device):
         super().__init__()
         self.dtype, self.device, self.layouts = dtype, device, {}
+        # namespace: the prefix the checkpoint's names carry; applied: tensors placed; converted:
+        # {"F32->bfloat16": count, ...} of those whose precision changed; aliased: stored names that
+        # are tied to an owner and were only compared with it; ignored: stored names the family
+        # lets be (legacy buffers)
+        self.report = {"namespace": "", "applied": 0, "converted": {}, "aliased": [], "ignored": []}
 
     def export(self):
         """The tensors back in checkpoint layout (float32, CPU), for tests and for saving."""
@@ -55,6 +61,10 @@ def place(store, spec, tensor):
         value = tensor.to(store.dtype).contiguous()
     store[spec.name] = value
     store.layouts[spec.name] = spec.layout
+    store.report["applied"] += 1
+    if value.dtype != tensor.dtype:
+        change = f"{str(tensor.dtype).replace('torch.', '')}->{str(value.dtype).replace('torch.', '')}"
+        store.report["converted"][change] = store.report["converted"].get(change, 0) + 1
 
 
 def store_from_tensors(tensors, contract, dtype, device, where="tensors"):
@@ -81,7 +91,7 @@ def load_checkpoint(model_dir, contract, dtype, device):
             if name in entries:
                 raise WeightError(model_dir, other=[f"tensor {name} is stored in two files"])
             entries[name] = entry
-    _, by_spec, stored_aliases = check(entries, contract, model_dir, listed - set(entries))
+    prefix, by_spec, stored_aliases = check(entries, contract, model_dir, listed - set(entries))
     reader = PayloadReader()
     try:
         for alias, owner in stored_aliases:        # before anything is placed on the device
@@ -96,4 +106,7 @@ def load_checkpoint(model_dir, contract, dtype, device):
             place(store, spec, reader.tensor(by_spec[spec.name]))
     finally:
         reader.close()
+    used = {prefix + spec.name for spec in contract.tensors} | {alias for alias, _ in stored_aliases}
+    store.report.update(namespace=prefix, aliased=sorted(alias for alias, _ in stored_aliases),
+                        ignored=sorted(set(entries) - used))
     return store

@@ -124,6 +124,10 @@ def test_namespaces_ignored_buffers_and_the_tied_head(tmp_path):
     assert store["h.0.ln_1.weight"].dtype == torch.float32
     exported = store.export()
     assert all(torch.equal(exported[k], tensors[k]) for k in tensors)
+    # what loading did is on record (src/checkpoint/report.rs:58-100)
+    assert store.report["namespace"] == "transformer." and store.report["applied"] == len(tensors)
+    assert store.report["aliased"] == ["lm_head.weight"] and store.report["converted"] == {}
+    assert store.report["ignored"] == ["transformer.h.0.attn.bias", "transformer.h.1.attn.masked_bias"]
     # a stored head that differs from the token table is refused
     prefixed["lm_head.weight"] = tensors["wte.weight"] + 1
     write_checkpoint(str(tmp_path / "untied"), prefixed)
@@ -164,6 +168,10 @@ def test_dtype_policy_and_sharded_checkpoints(tmp_path):
     assert store["ln_f.bias"].dtype == torch.float32                    # vectors always in float32
     rounded = tensors["h.0.mlp.c_fc.weight"].to(torch.bfloat16)         # one rounding to nearest even
     assert torch.equal(store["h.0.mlp.c_fc.weight"], rounded.t())
+    matrices = [k for k in names if tensors[k].dim() == 2]
+    assert store.report["converted"] == {"float32->bfloat16": sum(k in names[:half] for k in matrices),
+                                         "bfloat16->float32": sum(k in names[half:] for k in names if k not in matrices)}
+    assert store.report["namespace"] == "" and store.report["aliased"] == [] and store.report["ignored"] == []
     wide = load_checkpoint(folder, contract, torch.float32, "cpu")
     assert wide["wte.weight"].dtype == torch.float32
     with pytest.raises(ValueError, match="bfloat16 or float32"):

@@ -573,17 +573,31 @@ kv_store_bf16_kernel(const bf16_t* __restrict__ k_rows, const bf16_t* __restrict
     for (int j = 1; j < 4; ++j)
       if (run == j && t + j < tokens && seqs[1 + i + j] == seq && poss[1 + i + j] == pos + j && ((pos + j) & 3) != 0)
         run = j + 1;
+    if (run == 4) {
+      // pos is a multiple of four: eight channels of the four tokens are four 16-byte loads, and
+      // transposed they are 64 consecutive bytes of the cache
+      for (int c = threadIdx.x * 8; c < width; c += 256 * 8) {
+        int head = c / hd, channel = c % hd;
+        int4v row[4], quads[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) row[j] = *reinterpret_cast<const int4v*>(v_rows + (int64_t)(t + j) * ld + c);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {      // channels 2k and 2k + 1 lie in word k of every row
+          unsigned a = row[0][k], b = row[1][k], d = row[2][k], e = row[3][k];
+          quads[k] = int4v{(int)((a & 0xffffu) | (b << 16)), (int)((d & 0xffffu) | (e << 16)),
+                           (int)((a >> 16) | (b & 0xffff0000u)), (int)((d >> 16) | (e & 0xffff0000u))};
+        }
+        int4v* to = reinterpret_cast<int4v*>(values + kv_block_base(kv, seq, pos, head) + value_offset(hd, pos, channel));
+#pragma unroll
+        for (int k = 0; k < 4; ++k) to[k] = quads[k];
+      }
+      continue;
+    }
     for (int c = threadIdx.x; c < width; c += 256) {
       int head = c / hd, channel = c % hd;
       int64_t base = kv_block_base(kv, seq, pos, head);     // the run lies in one block
-      if (run == 4) {                                       // then pos is a multiple of four
-        bf16x4 quad = {v_rows[(int64_t)t * ld + c], v_rows[(int64_t)(t + 1) * ld + c],
-                       v_rows[(int64_t)(t + 2) * ld + c], v_rows[(int64_t)(t + 3) * ld + c]};
-        *reinterpret_cast<bf16x4*>(values + base + value_offset(hd, pos, channel)) = quad;
-      } else {
-        for (int j = 0; j < run; ++j)
-          values[base + value_offset(hd, pos + j, channel)] = v_rows[(int64_t)(t + j) * ld + c];
-      }
+      for (int j = 0; j < run; ++j)
+        values[base + value_offset(hd, pos + j, channel)] = v_rows[(int64_t)(t + j) * ld + c];
     }
   }
 }
@@ -595,7 +609,8 @@ BT_EXPORT int bt_kv_copy(void* stream, int dtype, void* k_rows, void* v_rows, in
   if (kv->head_dim <= 0 || kv->head_dim % 4 != 0) BT_REFUSE("kv_copy: head size %d must be a multiple of 4", kv->head_dim);
   dim3 grid(tokens), block(256);
   const bool wide = dtype != 0 && to_cache && tokens > 64 && kv->head_dim % 8 == 0 && ld % 8 == 0 &&
-                    ((uintptr_t)k_rows & 15) == 0 && ((uintptr_t)kv->keys & 15) == 0 && ((uintptr_t)kv->values & 7) == 0;
+                    ((uintptr_t)k_rows & 15) == 0 && ((uintptr_t)v_rows & 15) == 0 && ((uintptr_t)kv->keys & 15) == 0 &&
+                    ((uintptr_t)kv->values & 15) == 0;
   if (wide) {
     hipLaunchKernelGGL(kv_store_bf16_kernel, dim3((tokens + 3) / 4), block, 0, (hipStream_t)stream, (const bf16_t*)k_rows,
                        (const bf16_t*)v_rows, ld, tok_seq, tok_pos, *kv, tokens);

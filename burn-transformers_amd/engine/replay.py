@@ -30,6 +30,10 @@ class Replay:
         entries, want = [], []
         for entry in record.get("entries", []):
             request = entry["id"]
+            if not entry["tokens"]:           # nothing to run for this request in this step
+                if entry.get("want"):
+                    raise ValueError(f"step {record['step']}: request {request!r} wants logits but brings no token")
+                continue
             if request not in self.slots:
                 self.slots[request] = self.engine.open()
             entries.append((self.slots[request], entry["tokens"]))

@@ -358,11 +358,11 @@ def test_attention_tiled_float32(q_heads, kv_heads, hd, totals, counts, window):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("totals,counts", [([5, 70], [5, 3]), ([130, 67, 9, 260], [130, 66, 2, 77]),
                                            ([300], [299])])
-def test_kv_copy_round_trip(dtype, totals, counts):
+@pytest.mark.parametrize("kv_heads,hd", [(3, 16), (41, 64)])      # the second: more than one round of 8 x 256 channels
+def test_kv_copy_round_trip(dtype, totals, counts, kv_heads, hd):
     """Rows written into the paged cache (a few tokens: element by element; a prompt in bfloat16: runs
     of four positions at a time, starting anywhere) come back unchanged, and nothing else is touched."""
     dt = DTYPES[dtype]
-    kv_heads, hd = 3, 16
     case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=4)
     before_k, before_v = case.read_back()
     gen = torch.Generator().manual_seed(8)

@@ -114,8 +114,9 @@ def test_replay_whole_tail_and_batches(name, dtype, lengths, tmp_path):
 
 def test_replay_steps_without_wanted_places_write_nothing(tmp_path):
     r = prompts_for("A", [50], seed=52)[0]
-    steps = [{"step": 0, "entries": [{"id": "x", "tokens": r[:30], "want": []}], "end": []},
-             {"step": 1, "entries": [{"id": "x", "tokens": r[30:], "want": [19]}], "end": ["x"]}]
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": r[:30], "want": []},
+                                     {"id": "idle", "tokens": [], "want": []}], "end": []},      # an entry that brings nothing
+             {"step": 1, "entries": [{"id": "x", "tokens": r[30:], "want": [19]}], "end": ["x", "idle"]}]
     out = replay("A", "float32", steps, tmp_path, max_tokens=64)
     assert list(out) == [1]
     compare("A", "float32", out[1], plain_logits("A", r)[-1:], "cache filled by a step nobody read")

@@ -19,4 +19,9 @@ struct AttnArgs {
   int max_count;        // most tokens any sequence brings in this step
   int window;           // 0 = all earlier keys
   float scale;
+  // Decode only: with splits > 1 the keys of every sequence are cut into that many runs, each run
+  // is a work-group of its own that leaves (output row, maximum, sum) in `partial`
+  // [n_seqs][q_heads][splits][head_dim + 2], and a second kernel joins them into `out`.
+  int splits;
+  float* partial;
 };

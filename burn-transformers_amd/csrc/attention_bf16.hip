@@ -555,6 +555,7 @@ attention_decode_kernel(AttnArgs a) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i16 = lane & 15, g = lane >> 4;
   const int seq = blockIdx.y, kv_head = blockIdx.x;
+  const int splits = a.splits > 1 ? a.splits : 1, split = blockIdx.z;
   const int group = a.q_heads / a.kv.kv_heads;
   float* sm_m = sm;                                   // [DECODE_WAVES][group]
   float* sm_l = sm + DECODE_WAVES * group;            // [DECODE_WAVES][group]
@@ -572,7 +573,8 @@ attention_decode_kernel(AttnArgs a) {
   const int* block_row = a.kv.blocks + (int64_t)seq * a.kv.max_blocks;
   const int last_entry = a.kv.max_blocks - 1;
   int early_block0 = 0, early_block1 = 0;
-  if (a.window == 0) {
+  const bool early = a.window == 0 && splits == 1;    // (a later run's first tiles depend on the position)
+  if (early) {
     int entry0 = (32 * wave) / BT_KV_BLOCK, entry1 = (32 * wave + stride) / BT_KV_BLOCK;
     early_block0 = block_row[entry0 < last_entry ? entry0 : last_entry];
     early_block1 = block_row[entry1 < last_entry ? entry1 : last_entry];
@@ -594,15 +596,19 @@ attention_decode_kernel(AttnArgs a) {
   if (a.window > 0 && pos - a.window + 1 > 0) lo = (pos - a.window + 1) & ~31;
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
-  const int first = lo + 32 * wave;
+  // the tiles of 32 keys from `lo` through the query's own position, cut into `splits` runs
+  const int tiles = (pos - lo) / 32 + 1, per_split = (tiles + splits - 1) / splits;
+  const int tile_begin = split * per_split;
+  const int tile_end = tile_begin + per_split < tiles ? tile_begin + per_split : tiles;
+  const int first = lo + 32 * (tile_begin + wave), end = lo + 32 * tile_end;
   // plane of the tile at kb: from the blocks fetched early where they apply, else from the table
   auto plane_of = [&](int kb, int j) {
-    int block = (a.window == 0 && j < 2) ? (j == 0 ? early_block0 : early_block1) : block_row[kb / BT_KV_BLOCK];
+    int block = (early && j < 2) ? (j == 0 ? early_block0 : early_block1) : block_row[kb / BT_KV_BLOCK];
     return ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
   };
   const float c = a.scale * LOG2_E;
   auto fetch = [&](TileOperands& into, int kb, int j) {
-    if (kb <= pos) {
+    if (kb < end) {
       int64_t plane = plane_of(kb, j);
       load_tile(into, keys + plane, values + plane, kb);
     }
@@ -613,7 +619,7 @@ attention_decode_kernel(AttnArgs a) {
   TileOperands current, next;
   fetch(next, first, 0);
   int j = 0;
-  for (int kb = first; kb <= pos; kb += stride, ++j) {
+  for (int kb = first; kb < end; kb += stride, ++j) {
     current = next;
     fetch(next, kb + stride, j + 1);
     attend(current, kb);
@@ -647,7 +653,37 @@ attention_decode_kernel(AttnArgs a) {
         den += sm_l[w * group + j] * f;
       }
     }
-    out[(int64_t)tok * a.ldo + (kv_head * group + j) * HD + channel] = (bf16_t)(den > 0.f ? num / den : 0.f);
+    if (splits == 1) {
+      out[(int64_t)tok * a.ldo + (kv_head * group + j) * HD + channel] = (bf16_t)(den > 0.f ? num / den : 0.f);
+    } else {     // this run's share, for attention_join_kernel
+      float* mine = a.partial + (((int64_t)seq * a.q_heads + kv_head * group + j) * splits + split) * (HD + 2);
+      mine[channel] = num;
+      if (channel == 0) {
+        mine[HD] = top;
+        mine[HD + 1] = den;
+      }
+    }
+  }
+}
+
+// Joins the runs of attention_decode_kernel: a work-group of one wave per (sequence, query head).
+__global__ void __launch_bounds__(64)
+attention_join_kernel(AttnArgs a) {
+  const int seq = blockIdx.x / a.q_heads, head = blockIdx.x % a.q_heads;
+  const float* runs = a.partial + ((int64_t)seq * a.q_heads + head) * a.splits * (HD + 2);
+  float top = -INFINITY;
+  for (int s = 0; s < a.splits; ++s) top = fmaxf(top, runs[s * (HD + 2) + HD]);
+  bf16_t* out = static_cast<bf16_t*>(a.out) + (int64_t)seq * a.ldo + head * HD;
+  for (int channel = threadIdx.x; channel < HD; channel += 64) {
+    float num = 0.f, den = 0.f;
+    if (top != -INFINITY) {
+      for (int s = 0; s < a.splits; ++s) {
+        float f = exp2f(runs[s * (HD + 2) + HD] - top);
+        num += runs[s * (HD + 2) + channel] * f;
+        den += runs[s * (HD + 2) + HD + 1] * f;
+      }
+    }
+    out[channel] = (bf16_t)(den > 0.f ? num / den : 0.f);
   }
 }
 
@@ -713,9 +749,17 @@ BT_EXPORT int bt_attention_decode_bf16(void* stream, const AttnArgs* args) {
     BT_REFUSE("attention_decode_bf16: at most 16 query heads per key/value head, got %d",
               args->q_heads / args->kv.kv_heads);
   if (args->n_tokens != args->n_seqs) BT_REFUSE("attention_decode_bf16: needs exactly one token per sequence");
-  dim3 grid(args->kv.kv_heads, args->n_seqs);
+  const int splits = args->splits > 1 ? args->splits : 1;
+  if (splits > 1 && !args->partial) BT_REFUSE("attention_decode_bf16: %d runs of keys need a place for their partial results", splits);
+  if (splits > 65535 || args->n_seqs > 65535) BT_REFUSE("attention_decode_bf16: %d sequences in %d runs are too many", args->n_seqs, splits);
+  dim3 grid(args->kv.kv_heads, args->n_seqs, splits);
   int group = args->q_heads / args->kv.kv_heads;
   size_t lds = (size_t)DECODE_WAVES * group * (HD + 2) * sizeof(float);
   hipLaunchKernelGGL(attention_decode_kernel, grid, dim3(DECODE_WAVES * 64), lds, (hipStream_t)stream, *args);
+  if (splits > 1) {
+    rc = bt_check_launch("attention_decode_bf16");
+    if (rc) return rc;
+    hipLaunchKernelGGL(attention_join_kernel, dim3((unsigned)args->n_seqs * args->q_heads), dim3(64), 0, (hipStream_t)stream, *args);
+  }
   return bt_check_launch("attention_decode_bf16");
 }

@@ -223,7 +223,13 @@ attention_f32_decode_kernel(AttnArgs a) {
   if (tid < hd) qs[tid] = q[tid];
   __syncthreads();
   const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
-  const int first_block = lo / BT_KV_BLOCK, last_block = pos / BT_KV_BLOCK;
+  int first_block = lo / BT_KV_BLOCK, last_block = pos / BT_KV_BLOCK;
+  const int splits = a.splits > 1 ? a.splits : 1, split = blockIdx.z;
+  if (splits > 1) {       // this work-group's run of the blocks (it may be empty)
+    const int per_split = (last_block - first_block + splits) / splits;
+    first_block += split * per_split;
+    last_block = first_block + per_split - 1 < last_block ? first_block + per_split - 1 : last_block;
+  }
   const float* keys = static_cast<const float*>(a.kv.keys);
   const float* values = static_cast<const float*>(a.kv.values);
   float run_max = -INFINITY, run_sum = 0.f, acc[CPT];
@@ -295,6 +301,7 @@ attention_f32_decode_kernel(AttnArgs a) {
   if (wave == 0) {
     float top = fmaxf(fmaxf(part_max[0], part_max[1]), fmaxf(part_max[2], part_max[3]));
     float* out = static_cast<float*>(a.out) + (int64_t)seq * a.ldo + head * hd;
+    float* mine = splits > 1 ? a.partial + (((int64_t)seq * a.q_heads + head) * splits + split) * (hd + 2) : nullptr;
 #pragma unroll
     for (int j = 0; j < CPT; ++j) {
       int channel = lane + 64 * j;
@@ -306,8 +313,37 @@ attention_f32_decode_kernel(AttnArgs a) {
         num = fmaf(part_acc[w][channel], f, num);
         den = fmaf(part_sum[w], f, den);
       }
-      out[channel] = den > 0.f ? num / den : 0.f;
+      if (splits == 1) {
+        out[channel] = den > 0.f ? num / den : 0.f;
+      } else {                                                      // this run's share, for attention_f32_join_kernel
+        mine[channel] = num;
+        if (channel == 0) {
+          mine[hd] = top;
+          mine[hd + 1] = den;
+        }
+      }
     }
+  }
+}
+
+// Joins the runs of attention_f32_decode_kernel: a work-group of one wave per (sequence, head).
+__global__ void __launch_bounds__(64)
+attention_f32_join_kernel(AttnArgs a) {
+  const int hd = a.kv.head_dim;
+  const int seq = blockIdx.x / a.q_heads, head = blockIdx.x % a.q_heads;
+  const float* runs = a.partial + ((int64_t)seq * a.q_heads + head) * a.splits * (hd + 2);
+  float top = -INFINITY;
+  for (int s = 0; s < a.splits; ++s) top = fmaxf(top, runs[s * (hd + 2) + hd]);
+  float* out = static_cast<float*>(a.out) + (int64_t)seq * a.ldo + head * hd;
+  for (int channel = threadIdx.x; channel < hd; channel += 64) {
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < a.splits; ++s) {                            // an empty run: maximum -inf, weight 0
+      float run_top = runs[s * (hd + 2) + hd];
+      float f = run_top == -INFINITY ? 0.f : expf(run_top - top);
+      num = fmaf(runs[s * (hd + 2) + channel], f, num);
+      den = fmaf(runs[s * (hd + 2) + hd + 1], f, den);
+    }
+    out[channel] = den > 0.f ? num / den : 0.f;
   }
 }
 
@@ -326,11 +362,19 @@ BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
   if (a.ldq % 4 != 0 || ((uintptr_t)a.q & 15) || ((uintptr_t)a.kv.keys & 15) || ((uintptr_t)a.kv.values & 15))
     BT_REFUSE("attention_f32: queries, keys and values are read 16 bytes at a time (row pitch %lld)", (long long)a.ldq);
   if (a.max_count == 1 && a.n_tokens == a.n_seqs) {      // a decode step: one token per sequence, in their order
-    dim3 grid(a.n_seqs, a.q_heads);
+    const int splits = a.splits > 1 ? a.splits : 1;
+    if (splits > 1 && !a.partial) BT_REFUSE("attention_f32: %d runs of keys need a place for their partial results", splits);
+    if (splits > 65535 || a.q_heads > 65535) BT_REFUSE("attention_f32: %d heads in %d runs are too many", a.q_heads, splits);
+    dim3 grid(a.n_seqs, a.q_heads, splits);
     if (hd <= 64)
       hipLaunchKernelGGL(attention_f32_decode_kernel<1>, grid, dim3(256), 0, (hipStream_t)stream, a);
     else
       hipLaunchKernelGGL(attention_f32_decode_kernel<2>, grid, dim3(256), 0, (hipStream_t)stream, a);
+    if (splits > 1) {
+      int rc = bt_check_launch("attention_f32");
+      if (rc) return rc;
+      hipLaunchKernelGGL(attention_f32_join_kernel, dim3((unsigned)a.n_seqs * a.q_heads), dim3(64), 0, (hipStream_t)stream, a);
+    }
     return bt_check_launch("attention_f32");
   }
   const int q_tiles = (a.max_count + F32_QUERIES - 1) / F32_QUERIES;

@@ -11,6 +11,8 @@ sections of one int32 buffer:
 import numpy as np
 import torch
 
+from ..cache.ledger import BLOCK
+
 
 def _align(n):
     return (n + 3) & ~3
@@ -58,6 +60,22 @@ class StepPlan:
             table[row, :len(blocks)] = blocks
         self.host = host
         self.new_lengths = {slot: start + count for slot, start, count in zip(slots, starts, counts)}
+        self.context_limit = min(context_limit(max(self.new_lengths.values())), max_blocks * BLOCK)
+
+
+SHORT_CONTEXT = 1024
+
+
+def context_limit(longest):
+    """The class of a step by its longest sequence: SHORT_CONTEXT tokens, then powers of two (and never
+    more than a sequence can hold).  Parts
+    that plan their work by the context (attention cuts long contexts into runs) plan for this
+    bound instead of the exact lengths, so that a step's kernels depend only on its class, and a
+    captured graph serves every step of the same class."""
+    limit = SHORT_CONTEXT
+    while limit < longest:
+        limit *= 2
+    return limit
 
 
 class Step:
@@ -75,6 +93,7 @@ class Step:
         self.pool = pool
         self.max_count = host_plan.max_count if host_plan is not None else 1
         self.decode = host_plan.decode if host_plan is not None else True
+        self.context_limit = host_plan.context_limit if host_plan is not None else SHORT_CONTEXT
         # host-side copies for parts that plan their own work (None while a graph is replayed)
         self.host = host_plan
 

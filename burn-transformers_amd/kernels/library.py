@@ -46,7 +46,8 @@ class AttnArgs(ctypes.Structure):
     _fields_ = [("q", _c_ptr), ("ldq", _c_i64), ("out", _c_ptr), ("ldo", _c_i64),
                 ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("seq_off", _c_ptr), ("seq_start", _c_ptr),
                 ("kv", KvView), ("q_heads", _c_int), ("n_tokens", _c_int), ("n_seqs", _c_int),
-                ("max_count", _c_int), ("window", _c_int), ("scale", _c_float)]
+                ("max_count", _c_int), ("window", _c_int), ("scale", _c_float), ("splits", _c_int),
+                ("partial", _c_ptr)]
 
 
 class NormOperand(ctypes.Structure):
@@ -371,8 +372,18 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0):
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
-                   scale, window=0):
-    return AttnArgs(q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0),
+                   scale, window=0, partial=None):
+    """``partial``: float32 [n_seqs * q_heads * runs, head_dim + 2] for a decode step whose keys are
+    cut into runs that separate work-groups take (long contexts in small batches)."""
+    splits = 1
+    if partial is not None:
+        splits = partial.shape[0] // (n_seqs * q_heads)
+        if partial.dtype != torch.float32 or not partial.is_contiguous() or partial.shape[1] != kv_view.head_dim + 2 \
+                or splits * n_seqs * q_heads != partial.shape[0]:
+            raise KernelError(f"attention: partial results of shape {tuple(partial.shape)} do not fit "
+                              f"{n_seqs} sequences of {q_heads} heads of {kv_view.head_dim}")
+    return AttnArgs(splits=splits, partial=partial.data_ptr() if partial is not None and splits > 1 else None,
+                    q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0),
                     tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), seq_off=seq_off.data_ptr(),
                     seq_start=seq_start.data_ptr(), kv=kv_view, q_heads=q_heads, n_tokens=q.shape[0],
                     n_seqs=n_seqs, max_count=max_count, window=window or 0, scale=scale)

@@ -8,7 +8,8 @@ heads*head_dim] with its bias.
 One step: the fused projection's epilogue writes the queries to a buffer and scatters the new
 keys and values straight into the cache at each token's position; the attention kernel then
 reads the cache (prefill: tiled, online softmax; decode: one query per head, keys split over
-the waves); the output projection adds into the residual stream.
+the waves, and long contexts of a small batch over several work-groups); the output projection
+adds into the residual stream.
 Formulas: src/attention.rs:481-513 (projections), src/attention/dispatch.rs:314-328, 365-367,
 390-406 (scaled scores, exclusion by -inf, 32-bit softmax), src/attention.rs:882-897 (merge and
 output projection).
@@ -16,8 +17,17 @@ output projection).
 
 from ..cache.storage import KVSpec
 from ..kernels import library as K
-from .base import Mixer
+from .base import Mixer, compute_units
 from .registry import register
+
+# A decode step cuts long contexts into runs that separate work-groups take and a second kernel
+# joins.  Measured at 25 heads of 64 (us per call, runs 1 / 2 / 4 / 8 / 16): bfloat16, one
+# sequence, 1,024 keys 9.1 / 9.4 / 9.6 / 11.5 / 15.2, 2,048 keys 14.5 / 12.2 / 10.9 / 12.4 / 16.8,
+# 8,192 keys 47.7 / 29.6 / 23.0 / 19.3 / 23.6; eight sequences (200 pairs of sequence and head
+# already) lose with any cut, 73 / 80 / 85 us at 8,192 keys.  So: no more work-groups than
+# compute units, at least RUN_BYTES of keys and values per run, and no cut below SPLIT_BYTES.
+SPLIT_BYTES = 384 << 10
+RUN_BYTES = 128 << 10
 
 
 @register("mixer", "attention")
@@ -51,6 +61,18 @@ class CausalSelfAttention(Mixer):
     def head_dims(self):
         return (self.head_dim,)
 
+    def decode_runs(self, step, device):
+        """Into how many runs a decode step's keys are cut: planned for the step's class of
+        context, not its exact lengths, so that every step of a class runs the same kernels."""
+        if not step.decode:
+            return 1
+        keys = min(step.context_limit, self.window + 32) if self.window else step.context_limit
+        pair_bytes = keys * self.head_dim * 2 * (2 if step.dtype_is_bf16 else 4)     # one head's keys and values
+        if pair_bytes <= SPLIT_BYTES:
+            return 1
+        pairs = step.n_seqs * self.kv_heads
+        return max(1, min(compute_units(device) // pairs, pair_bytes // RUN_BYTES, 64))
+
     def forward(self, h, step, memory, stream):
         tokens = h.shape[0]
         kv = memory.kv()
@@ -71,7 +93,10 @@ class CausalSelfAttention(Mixer):
             bias = self.qkv_bias[:self.n_q] if self.qkv_bias is not None else None
             K.gemm(h, self.qkv_weight[:self.n_q], K.epilogue_store(q, bias))
         mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
+        partial, runs = None, self.decode_runs(step, h.device)
+        if runs > 1:
+            partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
-                                self.heads, step.n_seqs, step.max_count, self.scale, self.window)
+                                self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial)
         K.attention(args, step.dtype, step.decode)
         stream.add_product(step, mixed, self.out_weight, self.out_bias)

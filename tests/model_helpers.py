@@ -20,7 +20,11 @@ TINY_B = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer":
 TINY_C = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 1, "n_embd": 32, "n_head": 2,
           "n_inner": 37, "vocab_size": 131, "n_positions": 80, "activation_function": "gelu_new",
           "layer_norm_epsilon": 1e-3, "scale_attn_by_inverse_layer_idx": False}
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# room for contexts of several thousand tokens: decode steps there cut the keys into runs
+TINY_L = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "n_embd": 96, "n_head": 3,
+          "n_inner": 128, "vocab_size": 211, "n_positions": 4300, "activation_function": "gelu_new",
+          "layer_norm_epsilon": 1e-5, "scale_attn_by_inverse_layer_idx": False}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "L": (TINY_L, 3)}
 
 _folders = {}
 

@@ -220,6 +220,27 @@ def test_long_decoding(dtype):
     check(torch.cat(rows), want, dtype, "long decode")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_over_contexts_of_thousands(dtype):
+    """With contexts this long a decode step cuts every sequence's keys into runs for separate
+    work-groups (a short sequence beside the long ones has empty runs); the steps come from graphs
+    of their own class of context, and crossing 4,096 tokens starts the next class."""
+    engine = engine_for("L", dtype, max_tokens=4352 + 2112 + 64, gain=2.0)
+    requests = prompts_for("L", [4110, 2070, 40], seed=33)
+    want = [plain_logits("L", r, 2.0) for r in requests]
+    decoded = 22
+    slots = [engine.open() for _ in requests]
+    rows = [[engine.step([(slot, r[:-decoded])]).clone()] for slot, r in zip(slots, requests)]
+    assert ("attention.partial", torch.float32) not in engine.pool.buffers
+    for i in range(decoded, 0, -1):
+        logits = engine.step([(slot, [r[-i]]) for slot, r in zip(slots, requests)])
+        for row, got in zip(rows, logits):
+            row.append(got[None].clone())
+    assert ("attention.partial", torch.float32) in engine.pool.buffers and engine.graph_replays >= decoded - 4
+    for r, got, full in zip(requests, rows, want):
+        check(torch.cat(got), full[len(r) - decoded - 1:], dtype, f"request of {len(r)} tokens")
+
+
 def test_graph_and_eager_decoding_agree_bitwise():
     ids = prompts_for("A", [40], seed=31)[0]
     outs = []

@@ -432,6 +432,50 @@ def test_attention_finds_one_far_key_among_hundreds():
             assert rel_err(out, want) < 1e-2, (target, impl, decode)
 
 
+@pytest.mark.parametrize("dtype,hd,window", [("bfloat16", 64, 0), ("bfloat16", 32, 0), ("bfloat16", 64, 3000),
+                                             ("float32", 64, 0), ("float32", 112, 0), ("float32", 48, 1500)])
+def test_attention_decode_in_runs(dtype, hd, window):
+    """Long contexts of a small batch cut into runs that separate work-groups take and a second
+    kernel joins: every number of runs gives the result of the undivided kernel, also where a run
+    is empty (a short sequence beside long ones), and a single dominant key is found in whichever
+    run it falls."""
+    dt = DTYPES[dtype]
+    q_heads, kv_heads = 4, 2
+    totals = [5000, 2100, 70, 4097, 1]
+    case = PagedCase(totals, [1] * len(totals), kv_heads, hd, dt, DEV, seed=21, poison=True)
+    gen = torch.Generator().manual_seed(22)
+    q = torch.randn(len(totals), q_heads * hd, generator=gen) * 0.3
+    # sequence 0: head 0 looks at key 4321 alone, head 3 at key 17; sequence 3: head 1 at its last block
+    targets = [(0, 0, 4321), (0, 3, 17), (3, 1, 4040)]
+    seq = torch.cat([torch.full((t,), s, dtype=torch.int32) for s, t in enumerate(totals)]).to(DEV)
+    pos = torch.cat([torch.arange(t, dtype=torch.int32) for t in totals]).to(DEV)
+    for s, head, key in targets:
+        channels = slice((head // 2) * hd, (head // 2) * hd + hd)
+        case.k_rows[s][:, channels] *= 0.05
+        case.k_rows[s][key, (head // 2) * hd + 3] = 8.0
+        q[s, head * hd:(head + 1) * hd] = 0.0
+        q[s, head * hd + 3] = 8.0
+    K.kv_copy(torch.cat(case.k_rows).to(DEV), torch.cat(case.v_rows).to(DEV), seq, pos, case.view(), True)
+    q = q.to(dt).to(DEV)
+    want = case.reference(q, q_heads, 1.0, window)
+    for s, head, key in targets:
+        if window == 0 or key > totals[s] - 1 - window:
+            value = case.v_rows[s][key, (head // 2) * hd:(head // 2) * hd + hd].double()
+            assert (want[s, head * hd:(head + 1) * hd] - value).abs().max() < 1e-3
+    impl = "mfma" if dtype == "bfloat16" else "tiled"
+    bound = 1.2e-2 if dtype == "bfloat16" else 3e-6
+    for runs in (1, 2, 5, 19, 64):
+        out = torch.full((len(totals), q_heads * hd), float("nan"), dtype=dt, device=DEV)
+        partial = torch.full((len(totals) * q_heads * runs, hd + 2), float("nan"), device=DEV) if runs > 1 else None
+        args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                                q_heads, len(totals), 1, 1.0, window, partial)
+        K.attention(args, dt, decode=True, impl=impl)
+        assert rel_err(out, want) < bound, runs
+    with pytest.raises(K.KernelError, match="do not fit"):
+        K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                         q_heads, len(totals), 1, 1.0, window, torch.zeros(7, hd + 2, device=DEV))
+
+
 @pytest.mark.parametrize("pattern", ["ramp", "jumps", "falling"])
 def test_attention_with_scores_that_rise_and_jump(pattern):
     """The running maximum is allowed to lag a little before sums are rescaled: scores that creep

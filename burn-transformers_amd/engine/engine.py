@@ -171,7 +171,8 @@ class Engine:
         return self.model.forward(step, self.cache)
 
     def _run_from_graph(self, plan, readout):
-        key = (plan.layout.key(), plan.max_count, readout, plan.context_limit)
+        # (parts plan decode steps by the class of context; steps with prompt tokens look the same in every class)
+        key = (plan.layout.key(), plan.max_count, readout, plan.context_limit if plan.decode else 0)
         held = self._graphs.pop(key, None)
         if held is not None and held["generation"] != self.pool.generation:
             held = None                                   # a workspace moved: the graph is stale

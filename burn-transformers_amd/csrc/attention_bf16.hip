@@ -18,9 +18,13 @@
 //                      32 queries (two MFMA column tiles, which share every key and value load)
 //                      and walks the keys up to its last query's position.  (Four column tiles
 //                      per wave were measured and were slower: they leave one wave per SIMD.)
-//   attention_decode   one token per sequence: one work-group per (key/value head, sequence);
-//                      the query heads sharing that head are the MFMA columns; eight waves
-//                      split the keys and meet in LDS.
+//                      Heads of 64 without a window: eight waves, keys and values through LDS,
+//                      each block of keys taken by one of two sets of waves
+//                      (attention_prefill_split_kernel).
+//   attention_decode   one token per sequence: one work-group per (key/value head, sequence)
+//                      and run of keys; the query heads sharing that head are the MFMA columns;
+//                      eight waves split the keys and meet in LDS; the runs of a long context
+//                      are joined by attention_join_kernel.
 
 #include "host.h"
 #include "attention.h"
@@ -396,8 +400,8 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 #if BT_HEAD_DIM == 64
 // The same for heads of 64 without a window, with the keys and values shared through LDS: a
 // block of 64 positions (8 KiB of keys, 8 KiB of values, each one contiguous plane of the cache)
-// is brought in ONCE per work-group, one or two 16-byte pieces per thread, while the block
-// before it is being multiplied; every wave then reads its MFMA operands from LDS.  With each
+// is brought in ONCE per work-group, one 16-byte piece of each per thread, while the blocks
+// before it are being multiplied; every wave then reads its MFMA operands from LDS.  With each
 // wave loading its own operands from memory the kernel was bound by what one compute unit can
 // pull (about 25 GB/s): the four or eight waves asked for the same bytes four or eight times.
 //   keys:   row r (128 bytes) keeps its 16-byte chunk c at c ^ ((r >> 1) & 7): the 16 lanes of
@@ -409,40 +413,51 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 #define SHARED_V_BYTES (16 * SHARED_V_GROUP)
 #define SHARED_STAGE (SHARED_K_BYTES + SHARED_V_BYTES)
 
-template <bool PAIRED>
-__global__ void __launch_bounds__((PAIRED ? 2 : 1) * PREFILL_WAVES * 64)
-attention_prefill_shared_kernel(AttnArgs a) {
-  constexpr int THREADS = (PAIRED ? 2 : 1) * PREFILL_WAVES * 64;
-  constexpr int PIECES = 512 / THREADS;   // 16-byte pieces of an 8 KiB plane per thread
+// The KEYS of a tile are divided between two sets of four waves:
+// a work-group takes ONE tile of 128 queries, both sets hold the same queries (a wave of each set
+// the same 32), a turn brings two blocks of 64 keys in, the first set multiplies the even block
+// and the second the odd one, and at the end the second set hands its running maxima, sums and
+// output rows to the first through LDS, lane to lane.  Against a late and an early tile paired in
+// one work-group (the form of attention_prefill_kernel, which this replaced here) the longest
+// chain is half as long (a tile that ends at position 1,024 walks 8 turns, not 16 blocks), and
+// every SIMD has two waves at work all the time instead of one for most of it.  The tiles are
+// numbered latest first over the whole grid, so that the short ones fill in behind the long
+// ones.  Measured at 25 heads: 2 x 1,024 tokens 29.3 -> 27.3 us, 2,048 tokens 50.2 -> 43.2 us,
+// 4 chunks of 256 tokens behind 768 28.4 -> 21.8 us; what is left is the softmax's own
+// arithmetic (32 exponentials per lane and block at a quarter of the VALU rate).
+#define SPLIT_TURN (2 * SHARED_STAGE)
+#define SPLIT_LDS_BYTES (2 * SPLIT_TURN)
+
+__global__ void __launch_bounds__(2 * PREFILL_WAVES * 64)
+attention_prefill_split_kernel(AttnArgs a) {
+  constexpr int THREADS = 2 * PREFILL_WAVES * 64;
+  static_assert(THREADS == 512, "one 16-byte piece of a block's keys and one of its values per thread");
   typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2][SHARED_STAGE];
+  extern __shared__ __attribute__((aligned(16))) unsigned char split_lds[];   // [2 turns][2 blocks][SHARED_STAGE]
   const int tid = threadIdx.x, lane = tid & 63;
-  int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int set = wave8 / PREFILL_WAVES, wave = wave8 % PREFILL_WAVES;
   const int i16 = lane & 15, g = lane >> 4;
-  // numbering of work-groups, pairing of tiles: as in attention_prefill_kernel
+  // work-groups that read the same keys and values lie on one XCD (as in attention_prefill_kernel);
+  // within an XCD the tiles come latest first, all (sequence, head) pairs of a rank together
   const int group = a.q_heads / a.kv.kv_heads;
   const int q_tiles = (a.max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES;
-  const int pairs = PAIRED ? (q_tiles + 1) / 2 : q_tiles;
+  const int units = a.n_seqs * a.kv.kv_heads, units_per_xcd = (units + 7) / 8;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int unit = (slot / (group * pairs)) * 8 + xcd;
-  if (unit >= a.n_seqs * a.kv.kv_heads) return;             // the whole work-group
-  const int within = slot % (group * pairs);
+  const int per_rank = units_per_xcd * group;
+  const int rank = slot / per_rank, inside = slot % per_rank;
+  const int unit = (inside / group) * 8 + xcd;
+  if (unit >= units) return;                                // the whole work-group
   const int seq = unit / a.kv.kv_heads, kv_head = unit % a.kv.kv_heads;
-  const int head = kv_head * group + within % group;
-  const int pair = within / group, late = q_tiles - 1 - pair;
+  const int head = kv_head * group + inside % group;
+  const int q_tile = q_tiles - 1 - rank;
   const int off = a.seq_off[seq], count = a.seq_off[seq + 1] - off, start = a.seq_start[seq];
-  // the blocks the work-group walks: up to the last query of its later tile that exists
-  const int first_tile = PAIRED && pair < late ? pair : late;   // the earlier tile of the two (or the only one)
-  if (first_tile * PREFILL_QUERIES >= count) return;            // the whole work-group: no query of this sequence here
-  const int last_tile = late * PREFILL_QUERIES < count ? late : first_tile;
-  const int reach = (last_tile + 1) * PREFILL_QUERIES < count ? (last_tile + 1) * PREFILL_QUERIES : count;
+  if (q_tile * PREFILL_QUERIES >= count) return;            // the whole work-group: this sequence is shorter
+  const int reach = (q_tile + 1) * PREFILL_QUERIES < count ? (q_tile + 1) * PREFILL_QUERIES : count;
   const int n_blocks = (start + reach + BT_KV_BLOCK - 1) / BT_KV_BLOCK;
-  // this wave's queries; a wave without any still moves its share of every block
-  const bool second = PAIRED && wave >= PREFILL_WAVES;
-  const int q_tile = second ? pair : late;
-  wave &= PREFILL_WAVES - 1;
+  const int n_turns = (n_blocks + 1) / 2;
   const int q0 = q_tile * PREFILL_QUERIES + wave * PREFILL_QUERIES_PER_WAVE;
-  const bool active = !(second && pair == late) && q0 < count;
+  const bool active = q0 < count;                           // (a wave without queries still moves its share of every block)
   const bf16_t* Q = static_cast<const bf16_t*>(a.q);
 
   int qpos[PREFILL_NQ], tok[PREFILL_NQ];
@@ -467,46 +482,47 @@ attention_prefill_shared_kernel(AttnArgs a) {
   const int hi = active ? start + last : 0;     // one past the position of this wave's last query
   const int valid_end = start + count;
   const float c = a.scale * LOG2_E;
-  const int whole_until = start + q0 + 1;       // tiles ending here or before are seen whole
+  const int whole_until = start + q0 + 1;       // blocks ending here or before are seen whole
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
 
-  int4v kreg[PIECES], vreg[PIECES];
-  auto fetch = [&](int block_index) {
-    int64_t plane = tile_plane(a, seq, kv_head, block_index * BT_KV_BLOCK);
+  int4v kreg[2], vreg[2];
+  auto fetch = [&](int turn) {
 #pragma unroll
-    for (int u = 0; u < PIECES; ++u) {
-      int piece = tid + u * THREADS;
-      kreg[u] = *reinterpret_cast<const int4v*>(keys + plane + piece * 8);
-      vreg[u] = *reinterpret_cast<const int4v*>(values + plane + piece * 8);
+    for (int b = 0; b < 2; ++b) {
+      int block_index = 2 * turn + b;
+      if (block_index >= n_blocks) block_index = n_blocks - 1;     // (read again, never multiplied)
+      int64_t plane = tile_plane(a, seq, kv_head, block_index * BT_KV_BLOCK);
+      kreg[b] = *reinterpret_cast<const int4v*>(keys + plane + tid * 8);
+      vreg[b] = *reinterpret_cast<const int4v*>(values + plane + tid * 8);
     }
   };
-  auto stash = [&](unsigned char* stage) {
+  auto stash = [&](unsigned char* turn_base) {
+    const int row = tid >> 3, chunk = tid & 7, grp = tid >> 5, within = tid & 31;
 #pragma unroll
-    for (int u = 0; u < PIECES; ++u) {
-      int piece = tid + u * THREADS;
-      int row = piece >> 3, chunk = piece & 7;
-      *reinterpret_cast<int4v*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4)) = kreg[u];
-      int grp = piece >> 5, inside = piece & 31;
-      *reinterpret_cast<int4v*>(stage + SHARED_K_BYTES + grp * SHARED_V_GROUP + inside * 16) = vreg[u];
+    for (int b = 0; b < 2; ++b) {
+      unsigned char* stage = turn_base + b * SHARED_STAGE;
+      *reinterpret_cast<int4v*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4)) = kreg[b];
+      *reinterpret_cast<int4v*>(stage + SHARED_K_BYTES + grp * SHARED_V_GROUP + within * 16) = vreg[b];
     }
   };
   fetch(0);
-  stash(lds[0]);
+  stash(split_lds);
   __syncthreads();
-  for (int j = 0; j < n_blocks; ++j) {
-    const bool more = j + 1 < n_blocks;
-    if (more) fetch(j + 1);
-    const unsigned char* stage = lds[j & 1];
-    const int kb = j * BT_KV_BLOCK;
-    if (kb < hi) {
+  for (int t = 0; t < n_turns; ++t) {
+    const bool more = t + 1 < n_turns;
+    if (more) fetch(t + 1);
+    const int block_index = 2 * t + set;
+    const int kb = block_index * BT_KV_BLOCK;
+    if (block_index < n_blocks && kb < hi) {
+      const unsigned char* stage = split_lds + (t & 1) * SPLIT_TURN + set * SHARED_STAGE;
       BlockOperands blk;
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
-          int row = 16 * t + i16, chunk = ks * 4 + g;
-          blk.k[t][ks] = *reinterpret_cast<const bf16x8*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
+          int row = 16 * kt + i16, chunk = ks * 4 + g;
+          blk.k[kt][ks] = *reinterpret_cast<const bf16x8*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
         }
 #pragma unroll
       for (int dt = 0; dt < ND; ++dt) {
@@ -520,22 +536,48 @@ attention_prefill_shared_kernel(AttnArgs a) {
       else
         attend_block<PREFILL_NQ, true>(blk, kb, valid_end, qpos, c, q, o, m, l);
     }
-    if (more) stash(lds[(j + 1) & 1]);
-    __syncthreads();   // block j + 1 is in place, and everyone is done with block j before it is overwritten
+    if (more) stash(split_lds + ((t + 1) & 1) * SPLIT_TURN);
+    __syncthreads();   // turn t + 1 is in place, and everyone is done with turn t before it is overwritten
   }
-  if (!active) return;
+  // The second set's results go to the first, lane to lane: value k of lane `lane` of wave `wave`
+  // at float (k * PREFILL_WAVES + wave) * 64 + lane (everyone is past the last turn's barrier).
+  float* hand = reinterpret_cast<float*>(split_lds);
+  constexpr int PER_QUERY = 2 + 4 * ND;
+  if (set == 1) {
+#pragma unroll
+    for (int nq = 0; nq < PREFILL_NQ; ++nq) {
+      const int k0 = nq * PER_QUERY;
+      hand[((k0 + 0) * PREFILL_WAVES + wave) * 64 + lane] = m[nq];
+      hand[((k0 + 1) * PREFILL_WAVES + wave) * 64 + lane] = l[nq];
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) hand[((k0 + 2 + 4 * dt + r) * PREFILL_WAVES + wave) * 64 + lane] = o[nq][dt][r];
+    }
+  }
+  __syncthreads();
+  if (set == 1 || !active) return;
   bf16_t* out = static_cast<bf16_t*>(a.out);
 #pragma unroll
   for (int nq = 0; nq < PREFILL_NQ; ++nq) {
-    float total = l[nq];
+    const int k0 = nq * PER_QUERY;
+    const float m_other = hand[((k0 + 0) * PREFILL_WAVES + wave) * 64 + lane];
+    const float l_other = hand[((k0 + 1) * PREFILL_WAVES + wave) * 64 + lane];
+    const float top = fmaxf(m[nq], m_other);                       // (the maxima are kept in powers of two)
+    const float mine = m[nq] == -INFINITY ? 0.f : exp2f(m[nq] - top);
+    const float theirs = m_other == -INFINITY ? 0.f : exp2f(m_other - top);
+    float total = l[nq] * mine + l_other * theirs;
     total += __shfl_xor(total, 16, 64);
     total += __shfl_xor(total, 32, 64);
     float inv = total > 0.f ? 1.0f / total : 0.f;
     if (qpos[nq] < 0) continue;
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt) {
-      bf16x4 packed = {(bf16_t)(o[nq][dt][0] * inv), (bf16_t)(o[nq][dt][1] * inv), (bf16_t)(o[nq][dt][2] * inv),
-                       (bf16_t)(o[nq][dt][3] * inv)};
+      float joined[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        joined[r] = (o[nq][dt][r] * mine + hand[((k0 + 2 + 4 * dt + r) * PREFILL_WAVES + wave) * 64 + lane] * theirs) * inv;
+      bf16x4 packed = {(bf16_t)joined[0], (bf16_t)joined[1], (bf16_t)joined[2], (bf16_t)joined[3]};
       *reinterpret_cast<bf16x4*>(out + (int64_t)tok[nq] * a.ldo + head * HD + dt * 16 + 4 * g) = packed;
     }
   }
@@ -723,11 +765,18 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
   if (groups > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: %lld work-groups are too many", (long long)groups);
   dim3 grid((unsigned)groups);
 #if BT_HEAD_DIM == 64
-  if (args->window == 0) {    // keys and values shared through LDS
-    if (paired)
-      hipLaunchKernelGGL(attention_prefill_shared_kernel<true>, grid, dim3(2 * PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);
-    else
-      hipLaunchKernelGGL(attention_prefill_shared_kernel<false>, grid, dim3(PREFILL_WAVES * 64), 0, (hipStream_t)stream, *args);
+  if (args->window == 0) {   // keys and values shared through LDS, a tile's keys on two sets of waves
+    static bool raised = false;                 // 72 KB: beyond what a kernel gets without asking
+    if (!raised) {
+      hipError_t err = hipFuncSetAttribute((const void*)attention_prefill_split_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)SPLIT_LDS_BYTES);
+      if (err != hipSuccess) BT_REFUSE("attention_prefill_bf16: cannot get %d bytes of LDS: %s", (int)SPLIT_LDS_BYTES, hipGetErrorString(err));
+      raised = true;
+    }
+    const int64_t split_groups = 8 * units_per_xcd * group * q_tiles;
+    if (split_groups > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: %lld work-groups are too many", (long long)split_groups);
+    hipLaunchKernelGGL(attention_prefill_split_kernel, dim3((unsigned)split_groups), dim3(2 * PREFILL_WAVES * 64), SPLIT_LDS_BYTES,
+                       (hipStream_t)stream, *args);
     return bt_check_launch("attention_prefill_bf16");
   }
 #endif

@@ -143,6 +143,16 @@ def ensure(name, verbose=True):
     return found if found else compile_module(name, verbose)
 
 
+def ensure_many(names, verbose=True, jobs=8):
+    """The same for several modules; those that have to be compiled are compiled side by side."""
+    from concurrent.futures import ThreadPoolExecutor
+    missing = [name for name in dict.fromkeys(names) if _find(name, _hash(name)) is None]
+    if len(missing) > 1:
+        with ThreadPoolExecutor(max_workers=min(jobs, len(missing))) as pool:
+            list(pool.map(lambda n: compile_module(n, verbose), missing))
+    return {name: ensure(name, verbose) for name in names}
+
+
 def build_all(verbose=True, jobs=8):
     """Compiles every module anew (the build check of the repository)."""
     from concurrent.futures import ThreadPoolExecutor

@@ -163,14 +163,20 @@ def require_gpu():
 
 def prepare(dtype, head_dims=()):
     """Builds and loads what a model of this dtype and these head sizes needs."""
-    _module("core")
-    _module("gemm_mfma")
+    names = ["core", "gemm_mfma"]
+    if dtype == torch.bfloat16:
+        if os.environ.get(PRODUCTS_ENV, "") != "own":
+            names.append("gemm_library")
+        names += [f"attention_bf16_hd{size}" for size in head_dims]
+    elif any(size <= 128 for size in head_dims):
+        names.append("attention_f32")
+    with _lock:
+        build.ensure_many(names)        # what is missing is compiled side by side
+    for name in names:
+        if name != "gemm_library":
+            _module(name)
     if dtype == torch.bfloat16:
         library_products()
-        for size in head_dims:
-            _module(f"attention_bf16_hd{size}")
-    elif any(size <= 128 for size in head_dims):
-        _module("attention_f32")
 
 
 # --- the vendor's GEMM library for steps with many rows ---------------------------------------

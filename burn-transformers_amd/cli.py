@@ -68,6 +68,8 @@ def main(argv=None):
                         help="first write MODEL_DIR from this configuration with random weights")
     parser.add_argument("--weights-seed", type=int, default=0)
     parser.add_argument("--json", action="store_true", help="print one JSON object per sequence")
+    parser.add_argument("--load-report", action="store_true",
+                        help="print to stderr what loading did with the checkpoint's tensors (one JSON object)")
     args, extra = parser.parse_known_args(argv)
     if extra or args.max_new_tokens == 0:
         print(USAGE, file=sys.stderr)
@@ -88,6 +90,8 @@ def main(argv=None):
         frequency_penalty=args.frequency_penalty, additive_penalty_scope=args.additive_penalty_scope,
         no_repeat_ngram_size=args.no_repeat_ngram_size, logit_bias=args.logit_bias)
     model = bt.load_model(args.model_dir, dtype=args.dtype)
+    if args.load_report:
+        print(json.dumps(model.load_report), file=sys.stderr)
     grows_to = lambda n: n + args.max_new_tokens if args.total_length is None else min(n + args.max_new_tokens, args.total_length)
     need = sum((grows_to(len(p)) + 63) // 64 * 64 for p in prompts)
     engine = bt.Engine(model, max_tokens=args.max_tokens or need)

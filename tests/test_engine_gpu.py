@@ -474,8 +474,11 @@ def test_command_line(capsys, tmp_path):
     folder, config, weights = model_folder("A", 6.0)
     prompts = prompts_for("A", [6, 13], seed=60)
     text = ";".join(",".join(str(t) for t in p) for p in prompts)
-    assert main([folder, text, "5", "--dtype", "float32", "--json"]) == 0
-    lines = [json.loads(line) for line in capsys.readouterr().out.strip().splitlines()]
+    assert main([folder, text, "5", "--dtype", "float32", "--json", "--load-report"]) == 0
+    captured = capsys.readouterr()
+    lines = [json.loads(line) for line in captured.out.strip().splitlines()]
+    report = json.loads([line for line in captured.err.splitlines() if line.startswith("{")][-1])
+    assert report["applied"] == len(weights) and report["namespace"] == "" and report["ignored"] == []
     assert [line["token_ids"] for line in lines] == [plain.greedy(p, weights, config, 5) for p in prompts]
     assert all(line["finish_reason"] == "Length" for line in lines)
     assert main([folder, text, "0"]) == 2 and main([folder, text, "3", "4"]) == 2

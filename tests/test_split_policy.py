@@ -35,3 +35,40 @@ def test_choices_at_measured_sizes():
     assert split_count(8, 50257, 1600) == 1
     # beyond 16 rows a work-group owns 32 columns, so there are half as many tiles to spread
     assert split_count(64, 1600, 6400) >= split_count(8, 1600, 6400)
+
+
+# --- the runs a decode step's keys are cut into, and the classes of context ---------------------
+
+def _runs(monkeypatch, n_seqs, context_limit, kv_heads=25, head_dim=64, bf16=True, window=0, decode=True, units=256):
+    from types import SimpleNamespace
+    from burn_transformers_amd.parts import attention
+    monkeypatch.setattr(attention, "compute_units", lambda device: units)
+    mixer = SimpleNamespace(kv_heads=kv_heads, head_dim=head_dim, window=window)
+    step = SimpleNamespace(decode=decode, context_limit=context_limit, dtype_is_bf16=bf16, n_seqs=n_seqs)
+    return attention.CausalSelfAttention.decode_runs(mixer, step, "cuda:0")
+
+
+def test_decode_runs_at_measured_sizes(monkeypatch):
+    # 25 heads of 64: bfloat16 is not cut at 1,024 keys, and best with 4 / 8 runs at 2,048 / 4,096
+    assert _runs(monkeypatch, 1, 1024) == 1
+    assert _runs(monkeypatch, 1, 2048) == 4
+    assert _runs(monkeypatch, 1, 4096) == 8
+    assert _runs(monkeypatch, 1, 8192) == 10           # no more work-groups than compute units
+    assert _runs(monkeypatch, 4, 8192) == 2
+    assert _runs(monkeypatch, 8, 8192) == 1            # 200 pairs of sequence and head fill the chip
+    assert _runs(monkeypatch, 64, 8192) == 1
+    # float32 holds twice the bytes per key
+    assert _runs(monkeypatch, 1, 1024, bf16=False) == 4
+    assert _runs(monkeypatch, 8, 1024, bf16=False) == 1
+    # a window bounds the keys a query reads; steps with prompt tokens are never cut
+    assert _runs(monkeypatch, 1, 8192, window=512) == 1
+    assert _runs(monkeypatch, 1, 8192, decode=False) == 1
+
+
+def test_context_classes():
+    from burn_transformers_amd.engine.step import StepPlan, context_limit
+    assert [context_limit(n) for n in (1, 1024, 1025, 2048, 2049, 5000)] == [1024, 1024, 2048, 2048, 4096, 8192]
+    plan = StepPlan([0, 1], [10, 3000], [1, 1], [5, 6], [0, 1], [[0], list(range(47))], 128)
+    assert plan.context_limit == 4096 and plan.decode
+    # never more than a sequence can hold (3 blocks of 64 tokens here)
+    assert StepPlan([0], [100], [1], [5], [0], [[0, 1]], 3).context_limit == 192

@@ -83,26 +83,34 @@ class Engine:
             raise StepError("a step needs at least one sequence")
         ledger = self.cache.ledger
         slots, starts, counts, ids = [], [], [], []
+        limit = min(self.model.max_positions, self.cache.max_sequence_length)
+        vocab = self.model.vocab_size
         for slot, tokens in entries:
             if not ledger.live(slot):
                 raise StepError(f"slot {slot} is not open")
-            if slot in slots:
-                raise StepError(f"slot {slot} appears twice in one step")
-            tokens = np.asarray(tokens, dtype=np.int64).reshape(-1)
-            if tokens.size == 0:
-                raise StepError(f"slot {slot} brings no token; leave idle sequences out of the step")
-            if tokens.min() < 0 or tokens.max() >= self.model.vocab_size:
-                raise StepError(f"token ids of slot {slot} lie in {tokens.min()}..={tokens.max()}, "
-                                f"expected token values in 0..{self.model.vocab_size}")
+            if type(tokens) is list and len(tokens) == 1 and type(tokens[0]) is int:
+                size, low, high = 1, tokens[0], tokens[0]      # a decode step's entry: no array is made for it
+                ids.append(tokens[0])
+            else:
+                tokens = np.asarray(tokens, dtype=np.int64).reshape(-1)
+                size = int(tokens.size)
+                if size == 0:
+                    raise StepError(f"slot {slot} brings no token; leave idle sequences out of the step")
+                low, high = int(tokens.min()), int(tokens.max())
+                ids.extend(tokens.tolist())
+            if low < 0 or high >= vocab:
+                raise StepError(f"token ids of slot {slot} lie in {low}..={high}, "
+                                f"expected token values in 0..{vocab}")
             start = ledger.lengths[slot]
-            limit = min(self.model.max_positions, self.cache.max_sequence_length)
-            if start + tokens.size > limit:
-                raise StepError(f"slot {slot} would reach {start + tokens.size} tokens, "
+            if start + size > limit:
+                raise StepError(f"slot {slot} would reach {start + size} tokens, "
                                 f"the limit is {limit}")
             slots.append(slot)
             starts.append(start)
-            counts.append(int(tokens.size))
-            ids.append(tokens)
+            counts.append(size)
+        if len(set(slots)) != len(slots):
+            twice = next(slot for slot in slots if slots.count(slot) > 1)
+            raise StepError(f"slot {twice} appears twice in one step")
         offsets = np.concatenate([[0], np.cumsum(counts)])
         if want is None:
             wanted = [int(offsets[i + 1] - 1) for i in range(len(entries))]
@@ -122,8 +130,7 @@ class Engine:
         except RuntimeError as error:
             raise StepError(str(error)) from error
         # block rows are read after the reservation, in `step`
-        return dict(slots=slots, starts=starts, counts=counts, ids=np.concatenate(ids), wanted=wanted,
-                    new_lengths=new_lengths)
+        return dict(slots=slots, starts=starts, counts=counts, ids=ids, wanted=wanted, new_lengths=new_lengths)
 
     def step(self, entries, want=None):
         """Runs one step; returns float32 logits [wanted places, vocab] on the GPU, valid until the

@@ -46,12 +46,16 @@ class StepPlan:
         self.decode = self.max_count == 1
         self.layout = StepLayout(self.n_tokens, self.n_seqs, len(wanted), max_blocks)
         host = np.zeros(self.layout.total, dtype=np.int32)
-        offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
         section = lambda name: host[self.layout.sections[name][0]:sum(self.layout.sections[name])]
         section("tok_ids")[:] = token_ids
-        section("tok_pos")[:] = np.concatenate([np.arange(s, s + c) for s, c in zip(starts, counts)])
-        section("tok_seq")[:] = np.repeat(np.arange(self.n_seqs), counts)
-        section("seq_off")[:] = offsets
+        if self.decode:          # one token each: a token's place in the step is its sequence's
+            section("tok_pos")[:] = starts
+            section("tok_seq")[:] = np.arange(self.n_seqs, dtype=np.int32)
+            section("seq_off")[:] = np.arange(self.n_seqs + 1, dtype=np.int32)
+        else:
+            section("tok_pos")[:] = np.concatenate([np.arange(s, s + c) for s, c in zip(starts, counts)])
+            section("tok_seq")[:] = np.repeat(np.arange(self.n_seqs), counts)
+            section("seq_off")[:] = np.concatenate([[0], np.cumsum(counts)])
         section("seq_start")[:] = starts
         section("slots")[:] = slots
         section("sel_rows")[:] = wanted

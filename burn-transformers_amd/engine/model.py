@@ -82,6 +82,43 @@ class CausalLM:
             return self.readout.logits(hidden, step)
 
 
+    # --- the short way round ----------------------------------------------------------------
+    @classmethod
+    def from_pretrained(cls, model_dir, dtype="bfloat16", device=None):
+        """``load_model`` under the name such loaders usually carry."""
+        return load_model(model_dir, dtype, device)
+
+    @classmethod
+    def random(cls, config_json, seed=0, dtype="bfloat16", device=None):
+        """A model with the random weights ``write_random_model`` writes for this seed (rounded to
+        bfloat16 as it stores them), without the folder."""
+        import torch
+        from ..weights.random_init import random_tensors
+        _, tensors = random_tensors(config_json, seed)
+        return model_from_tensors(config_json, {k: v.to(torch.bfloat16) for k, v in tensors.items()}, dtype, device)
+
+    def engine(self, max_tokens, **options):
+        """An engine (cache and step function) for this model."""
+        from .engine import Engine
+        return Engine(self, max_tokens, **options)
+
+    def generate(self, prompts, config=None, max_tokens=None, **options):
+        """Generates for the prompts with an engine whose cache is as large as they need (or
+        ``max_tokens``); see ``engine.generate.generate`` for the options."""
+        from ..cache.ledger import BLOCK
+        from ..sampling.config import GenerationConfig
+        from .generate import generate
+        config = config or GenerationConfig()
+        if max_tokens is None:
+            grows_to = lambda n: min(n + config.max_new_tokens, options.get("total_length") or self.max_positions)
+            max_tokens = sum((grows_to(len(p)) + BLOCK - 1) // BLOCK * BLOCK for p in prompts)
+        return generate(self.engine(max_tokens), prompts, config, **options)
+
+    def export_weights(self):
+        """The tensors back under their checkpoint names and layouts (float32, CPU)."""
+        return self.store.export()
+
+
 def _device(device):
     import torch
     K.require_gpu()

@@ -408,6 +408,21 @@ def test_greedy_generation_through_the_entry_point(name):
     engine.cache.ledger.check()
 
 
+def test_the_short_way_round_model_random_generate_export():
+    """CausalLM.random gives the model that the written folder loads to; model.generate sizes its own
+    cache; export_weights gives the stored tensors back."""
+    folder, config, weights = model_folder("B")
+    model = bt.CausalLM.random(config, seed=CONFIGS["B"][1], dtype="float32")
+    exported = model.export_weights()
+    assert set(exported) == set(weights) and all(torch.equal(exported[k], weights[k]) for k in weights)
+    prompts = prompts_for("B", [4, 30], seed=44)
+    got = model.generate(prompts, bt.GenerationConfig(max_new_tokens=6))
+    loaded = bt.CausalLM.from_pretrained(folder, dtype="float32")
+    same = bt.generate(loaded.engine(max_tokens=256), prompts, bt.GenerationConfig(max_new_tokens=6))
+    assert [s.token_ids for s in got] == [s.token_ids for s in same]
+    assert [s.token_ids for s in got] == [plain.greedy(p, weights, config, 6) for p in prompts]
+
+
 def test_unequal_prompts_grown_to_the_position_limit():
     """Prompts of 5, 100 and 127 tokens all decoded to the model's 128 positions in one batch: each
     ends by its own length, the long ones first, and the tokens are the plain greedy loop's."""

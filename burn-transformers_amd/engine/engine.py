@@ -27,7 +27,6 @@ import numpy as np
 import torch
 
 from ..cache.storage import Cache
-from .stack import DecodeStack
 from .step import BufferPool, Step, StepLayout, StepPlan
 
 _PINNED_RING = 4
@@ -39,14 +38,12 @@ class StepError(ValueError):
 
 
 class Engine:
-    def __init__(self, model, max_tokens, max_slots=None, graphs=True, stack=True):
+    def __init__(self, model, max_tokens, max_slots=None, graphs=True):
         self.model = model
         self.device, self.dtype = model.device, model.dtype
         self.cache = Cache(model.kv_specs, model.state_specs, max_tokens, model.max_positions,
                            model.dtype, model.device, max_slots)
         self.pool = BufferPool(self.device)
-        # small decode steps of a model whose layers are all of one arrangement run as one kernel
-        self.stack = DecodeStack.build(model, self.cache) if stack else None
         # a mixer that plans work on the host per step cannot be replayed from a graph
         self.use_graphs = graphs and all(getattr(block.parts.get("mixer"), "graph_safe", True)
                                          for block in model.blocks)
@@ -65,8 +62,6 @@ class Engine:
 
     def close(self, slot):
         """Ends a sequence: its slot and its blocks can be used again."""
-        if self.stack is not None:
-            self.stack.check(force=True)
         self.cache.release(slot)
 
     def length(self, slot):
@@ -155,8 +150,6 @@ class Engine:
         for slot, length in checked["new_lengths"].items():
             ledger.commit(slot, length)
         self.steps_run += 1
-        if self.stack is not None:
-            self.stack.check()
         return logits
 
     # --- running ---------------------------------------------------------------------------
@@ -180,9 +173,9 @@ class Engine:
         self._upload(plan.host, self._meta)
         step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
         if not want_logits:       # a step whose logits nobody wants still has to fill the cache
-            self.model.forward(step, self.cache, readout=False, stack=self.stack)
+            self.model.forward(step, self.cache, readout=False)
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
-        return self.model.forward(step, self.cache, stack=self.stack)
+        return self.model.forward(step, self.cache)
 
     def _run_from_graph(self, plan, readout):
         # (parts plan decode steps by the class of context; steps with prompt tokens look the same in every class)
@@ -216,7 +209,7 @@ class Engine:
         self.pool.frozen = True
         try:
             with torch.cuda.graph(graph):
-                logits = self.model.forward(step, self.cache, readout=readout, stack=self.stack)
+                logits = self.model.forward(step, self.cache, readout=readout)
         finally:
             self.pool.frozen = False
         if not readout:

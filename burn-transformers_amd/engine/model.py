@@ -68,16 +68,14 @@ class CausalLM:
         self.kv_specs = [writers.get(i, (None, None))[0] for i in range(self.cache_entries)]
         self.state_specs = [writers.get(i, (None, None))[1] for i in range(self.cache_entries)]
 
-    def forward(self, step, cache, readout=True, stack=None):
+    def forward(self, step, cache, readout=True):
         """Logits (float32 [len(step.sel_rows), vocab]) of the step's wanted rows; with
-        ``readout=False`` the layers only fill the cache and nothing is returned.  ``stack``: the
-        engine's one-kernel form of the whole schedule (``engine/stack.py``), used for the steps it takes."""
+        ``readout=False`` the layers only fill the cache and nothing is returned."""
         with K.one_stream():          # the hundreds of launches below ask for the current stream once
             stream = self.embedding.embed(step)
-            if stack is None or not stack.takes(step) or not stack.run(stream, step):
-                for entry in self.schedule:
-                    memory = Memory(cache, entry.cache, entry.writes, step) if entry.cache is not None else None
-                    self.blocks[entry.layer].forward(stream, step, memory)
+            for entry in self.schedule:
+                memory = Memory(cache, entry.cache, entry.writes, step) if entry.cache is not None else None
+                self.blocks[entry.layer].forward(stream, step, memory)
             if not readout:
                 return None
             hidden = self.final_norm.apply(stream, step, rows=step.sel_rows)

@@ -19,7 +19,7 @@ import time
 PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
-HEADERS = ("common.h", "host.h", "epilogue.h", "attention.h", "attention_tile.h")
+HEADERS = ("common.h", "host.h", "epilogue.h", "attention.h")
 # -packed-fp32-ops is switched off for every kernel: some packed 32-bit forms have produced
 # wrong values on this hardware generation.
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=" + ARCH, "-fPIC", "-shared",
@@ -36,11 +36,6 @@ def module_source(name):
                 f"no bfloat16 attention kernel for head size {size}: "
                 f"sizes {ATTENTION_HEAD_SIZES[0]}..{ATTENTION_HEAD_SIZES[-1]} in steps of 16 are built")
         return "attention_bf16.hip", [f"-DBT_HEAD_DIM={size}"]
-    if name.startswith("decode_stack_hd"):
-        size = int(name[len("decode_stack_hd"):])
-        if size not in ATTENTION_HEAD_SIZES:
-            raise ValueError(f"no layer-stack kernel for head size {size}")
-        return "decode_stack.hip", [f"-DBT_HEAD_DIM={size}"]
     if name in ("core", "gemm_mfma", "attention_f32"):
         return name + ".hip", []
     if name == "gemm_library":      # host code around hipBLASLt, which it opens at run time
@@ -49,8 +44,7 @@ def module_source(name):
 
 
 def all_modules():
-    return (["core", "gemm_mfma", "gemm_library", "attention_f32"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
-            + [f"decode_stack_hd{s}" for s in ATTENTION_HEAD_SIZES])
+    return ["core", "gemm_mfma", "gemm_library", "attention_f32"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
 
 
 def _hash(name):

@@ -55,24 +55,6 @@ class NormOperand(ctypes.Structure):
                 ("kind", _c_int)]
 
 
-class StackLayer(ctypes.Structure):
-    """One layer of a pre-norm stack as the one-kernel decode step reads it (a device array of these)."""
-    _fields_ = [("norm1_scale", _c_ptr), ("norm1_shift", _c_ptr), ("norm2_scale", _c_ptr), ("norm2_shift", _c_ptr),
-                ("qkv_weight", _c_ptr), ("qkv_bias", _c_ptr), ("out_weight", _c_ptr), ("out_bias", _c_ptr),
-                ("up_weight", _c_ptr), ("up_bias", _c_ptr), ("down_weight", _c_ptr), ("down_bias", _c_ptr),
-                ("keys", _c_ptr), ("values", _c_ptr), ("eps1", _c_float), ("eps2", _c_float),
-                ("scale", _c_float), ("reserved", _c_int)]
-
-
-class StackArgs(ctypes.Structure):
-    _fields_ = [("layers", _c_ptr), ("n_layers", _c_int), ("rows", _c_int), ("x", _c_ptr), ("ldx", _c_i64),
-                ("width", _c_int), ("inner", _c_int), ("heads", _c_int), ("kv_heads", _c_int),
-                ("norm_kind", _c_int), ("act", _c_int), ("window", _c_int), ("max_blocks", _c_int),
-                ("cols_qkv", _c_int), ("cols_up", _c_int), ("cols_x", _c_int),
-                ("blocks", _c_ptr), ("positions", _c_ptr), ("q", _c_ptr), ("mixed", _c_ptr), ("hidden", _c_ptr),
-                ("between", _c_ptr), ("sync", _c_ptr), ("clocks", _c_ptr)]
-
-
 class Normalized:
     """Rows of the float32 residual stream that are still to be normalised: handed to ``gemm`` in
     place of its activations, the skinny product kernel normalises them itself (up to 16 rows of
@@ -108,7 +90,6 @@ _SIGNATURES = {
     "bt_attention_f32": [_c_ptr, _P(AttnArgs)],
     "bt_attention_prefill_bf16": [_c_ptr, _P(AttnArgs)],
     "bt_attention_decode_bf16": [_c_ptr, _P(AttnArgs)],
-    "bt_decode_stack": [_c_ptr, _P(StackArgs), _c_int],
     "bt_kv_copy": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _P(KvView), _c_int, _c_int],
 }
 
@@ -187,7 +168,6 @@ def prepare(dtype, head_dims=()):
         if os.environ.get(PRODUCTS_ENV, "") != "own":
             names.append("gemm_library")
         names += [f"attention_bf16_hd{size}" for size in head_dims]
-        names += [f"decode_stack_hd{size}" for size in head_dims if size <= 128]    # (see engine/stack.py)
     elif any(size <= 128 for size in head_dims):
         names.append("attention_f32")
     with _lock:
@@ -440,27 +420,6 @@ def attention(args, dtype, decode, impl="auto"):
     lib = _module(f"attention_bf16_hd{args.kv.head_dim}")
     fn = lib.bt_attention_decode_bf16 if decode else lib.bt_attention_prefill_bf16
     _check(lib, fn(_stream(), args))
-
-
-STACK_MAX_ROWS = 16
-
-
-def decode_stack_module(head_dim):
-    """The one-kernel decode step for this head size (built when first asked for)."""
-    return _module(f"decode_stack_hd{head_dim}")
-
-
-def decode_stack_sync(head_dim, device):
-    """(zeroed int32 tensor for the kernel's barrier, index of the word it sets when a wait gave up)."""
-    lib = decode_stack_module(head_dim)
-    return (torch.zeros(lib.bt_decode_stack_sync_words(), dtype=torch.int32, device=device),
-            lib.bt_decode_stack_failed_word())
-
-
-def decode_stack(head_dim, args, grid):
-    """Launches the kernel; the barrier's words must be zero (``sync.zero_()`` on the same stream)."""
-    lib = decode_stack_module(head_dim)
-    _check(lib, lib.bt_decode_stack(_stream(), ctypes.byref(args), grid))
 
 
 def kv_copy(k_rows, v_rows, tok_seq, tok_pos, kv_view, to_cache):

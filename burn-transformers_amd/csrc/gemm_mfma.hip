@@ -498,7 +498,7 @@ __device__ float bt_norm_zeros[4] = {0.f, 0.f, 0.f, 0.f};
 template <typename T, int MT, int NT, int U, int WAVES, int QPL = 0>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W, int M, int N,
-                   int K, Epilogue epi, int tile_columns, NormOperand norm) {
+                   int K, Epilogue epi, int tile_columns, NormOperand norm, int packed) {
   constexpr int ELEMS = Mma<T>::ELEMS;      // K values in a lane's 16-byte load
   constexpr int CHUNK = 4 * ELEMS;          // K values the wave's four K groups cover together
   constexpr bool NORM = QPL > 0;
@@ -518,11 +518,18 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
   const int n_base = blockIdx.x * tile_columns;
   const int n_end = n_base + tile_columns < N ? n_base + tile_columns : N;   // one past this work-group's last column
   const int split = blockIdx.y, splits = gridDim.y;
+  // packed: W is not [N][K] but, for each work-group's `tile_columns` columns, the chunks of K one
+  // after the other, [group][chunk][tile_columns][CHUNK], K and the last group padded with zeros:
+  // a wave's load of a chunk is then one contiguous run of bytes and a work-group reads one
+  // contiguous block front to back.
+  const int w_chunk_pitch = packed ? tile_columns * CHUNK : CHUNK;     // elements from one chunk to the next
   const T* w_row[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     int n = n_base + nt * 16 + i16;
-    w_row[nt] = W + (int64_t)(n < n_end ? n : n_end - 1) * K;
+    n = n < n_end ? n : n_end - 1;
+    w_row[nt] = packed ? W + ((int64_t)blockIdx.x * ((K + CHUNK - 1) / CHUNK) * tile_columns + (n - n_base)) * CHUNK
+                       : W + (int64_t)n * K;
   }
   const T* a_row[MT];
 #pragma unroll
@@ -555,8 +562,9 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
       if (cc < chunks) {
         int k = cc * CHUNK + g * ELEMS;
         int kc = k < K ? k : K - ELEMS;
+        int wc = packed ? cc * w_chunk_pitch + g * ELEMS : kc;      // (the packed chunks are whole: zeros beyond K)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wv[u][nt] = *reinterpret_cast<const int4v*>(w_row[nt] + kc);
+        for (int nt = 0; nt < NT; ++nt) wv[u][nt] = *reinterpret_cast<const int4v*>(w_row[nt] + wc);
         if constexpr (!NORM) {
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + kc);
@@ -760,11 +768,11 @@ BT_EXPORT int bt_gemm_tile(void* stream, int dtype, const void* A, int64_t lda, 
 
 template <typename T>
 static void launch_skinny(hipStream_t s, const T* a, int64_t lda, const T* w, int M, int N, int K, const Epilogue& epi,
-                          int splits, int columns) {
+                          int splits, int columns, int packed) {
   dim3 grid((N + columns - 1) / columns, splits), block(512);
   const NormOperand none = {};
 #define LAUNCH_SKINNY(MT, NT, U) \
-  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns, none)
+  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns, none, packed)
   if (M <= 16) {
     if (columns <= 16) LAUNCH_SKINNY(1, 1, 8); else LAUNCH_SKINNY(1, 2, 8);
   } else if (M <= 32) {
@@ -778,7 +786,7 @@ static void launch_skinny(hipStream_t s, const T* a, int64_t lda, const T* w, in
 // The product of the normalised rows of a float32 residual stream (see NormOperand): bfloat16
 // weights, up to 16 rows, K up to 2048 and a multiple of 8.
 static int launch_skinny_norm(hipStream_t s, const NormOperand& norm, const bf16_t* w, int M, int N, int K,
-                              const Epilogue& epi, int splits, int columns) {
+                              const Epilogue& epi, int splits, int columns, int packed) {
   dim3 grid((N + columns - 1) / columns, splits), block(512);
   size_t lds = (size_t)16 * (K * 2 + 16);
 #define LAUNCH_NORM(NT, QPL)                                                                                   \
@@ -790,7 +798,7 @@ static int launch_skinny_norm(hipStream_t s, const NormOperand& norm, const bf16
       if (err != hipSuccess) BT_REFUSE("gemm_skinny: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));   \
       granted = lds;                                                                                           \
     }                                                                                                          \
-    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)nullptr, (int64_t)0, w, M, N, K, epi, columns, norm); \
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)nullptr, (int64_t)0, w, M, N, K, epi, columns, norm, packed); \
   } while (0)
   if (K <= 1024) {
     if (columns <= 16) LAUNCH_NORM(1, 4); else LAUNCH_NORM(2, 4);
@@ -802,8 +810,10 @@ static int launch_skinny_norm(hipStream_t s, const NormOperand& norm, const bf16
 }
 
 // norm: null, or the activations are the normalised rows it describes (then A and lda are ignored)
+// packed_columns: 0, or W is the packed form of the matrix for that many columns per work-group (see
+// the kernel), which then is the number of columns a work-group takes.
 BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                             const Epilogue* epi, int splits, int variant, const NormOperand* norm) {
+                             const Epilogue* epi, int splits, int variant, const NormOperand* norm, int packed_columns) {
   if (M <= 0) return BT_OK;
   if (M > 64) BT_REFUSE("gemm_skinny: %d rows, at most 64", M);
   if (dtype != 0 && dtype != 1) BT_REFUSE("gemm_skinny: element type %d is neither float nor bfloat16", dtype);
@@ -832,7 +842,12 @@ BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda
   // columns per work-group: the cost of a work-group is what it pulls for one chunk of K (its
   // columns of the weights and the step's rows of the activations) times its chunks, plus a fixed part
   int columns = M <= 16 ? 16 : 32;
-  if (variant >= 8 && variant <= 32 && variant % 4 == 0) {
+  const int packed = packed_columns != 0;
+  if (packed) {
+    if (packed_columns < 8 || packed_columns > 32 || packed_columns % 4 != 0)
+      BT_REFUSE("gemm_skinny: a matrix packed for %d columns per work-group (8, 12, ... 32 are possible)", packed_columns);
+    columns = packed_columns;
+  } else if (variant >= 8 && variant <= 32 && variant % 4 == 0) {
     columns = variant;
   } else if (variant == 0) {
     const int chunk = 4 * elems;
@@ -845,12 +860,12 @@ BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda
     }
   }
   if (norm != nullptr) {
-    rc = launch_skinny_norm((hipStream_t)stream, *norm, (const bf16_t*)W, M, N, K, *epi, splits, columns);
+    rc = launch_skinny_norm((hipStream_t)stream, *norm, (const bf16_t*)W, M, N, K, *epi, splits, columns, packed);
     if (rc) return rc;
   } else if (dtype == 0) {
-    launch_skinny<float>((hipStream_t)stream, (const float*)A, lda, (const float*)W, M, N, K, *epi, splits, columns);
+    launch_skinny<float>((hipStream_t)stream, (const float*)A, lda, (const float*)W, M, N, K, *epi, splits, columns, packed);
   } else {
-    launch_skinny<bf16_t>((hipStream_t)stream, (const bf16_t*)A, lda, (const bf16_t*)W, M, N, K, *epi, splits, columns);
+    launch_skinny<bf16_t>((hipStream_t)stream, (const bf16_t*)A, lda, (const bf16_t*)W, M, N, K, *epi, splits, columns, packed);
   }
   return bt_check_launch("gemm_skinny");
 }

@@ -17,7 +17,7 @@ output projection).
 
 from ..cache.storage import KVSpec
 from ..kernels import library as K
-from .base import Mixer, compute_units
+from .base import Mixer, compute_units, packed_for_stream
 from .registry import register
 
 # A decode step cuts long contexts into runs that separate work-groups take and a second kernel
@@ -55,6 +55,10 @@ class CausalSelfAttention(Mixer):
             raise ValueError(f"attention: output projection is {tuple(self.out_weight.shape)}, "
                              f"expected {(self.width, self.n_q)}")
 
+        # second copies for decode steps, which read the weights and little else
+        self.qkv_packed = K.PackedWeight(self.qkv_weight) if self.qkv_weight.is_cuda else None
+        self.out_packed = packed_for_stream(self.out_weight) if self.out_weight.is_cuda else None
+
     def kv_spec(self):
         return KVSpec(self.kv_heads, self.head_dim, self.window)
 
@@ -87,7 +91,8 @@ class CausalSelfAttention(Mixer):
         elif memory.writes:
             q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
             K.gemm(h, self.qkv_weight,
-                   K.epilogue_qkv(q, self.n_q, self.n_kv, kv, step.tok_seq, step.tok_pos, self.qkv_bias))
+                   K.epilogue_qkv(q, self.n_q, self.n_kv, kv, step.tok_seq, step.tok_pos, self.qkv_bias),
+                   packed=self.qkv_packed)
         else:   # the keys and values of another layer are read; only the queries are projected
             q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
             bias = self.qkv_bias[:self.n_q] if self.qkv_bias is not None else None
@@ -99,4 +104,4 @@ class CausalSelfAttention(Mixer):
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                 self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial)
         K.attention(args, step.dtype, step.decode)
-        stream.add_product(step, mixed, self.out_weight, self.out_bias)
+        stream.add_product(step, mixed, self.out_weight, self.out_bias, packed=self.out_packed)

@@ -48,11 +48,11 @@ class ResidualStream:
             self.flush()
         self.pending = delta
 
-    def add_product(self, step, a, weight, bias=None):
+    def add_product(self, step, a, weight, bias=None, packed=None):
         """x += a . weight^T + bias.  In a decode step (up to 64 rows) a product with few
         output columns splits its K range into partial sums that stay pending: the extra work-groups
         are needed to pull the matrix through HBM.  Otherwise the product's epilogue adds into the
-        stream in place."""
+        stream in place.  ``packed``: the weight's ``kernels.library.PackedWeight``, if it has one."""
         rows, width = a.shape[0], weight.shape[0]
         if self.in_place:
             splits = 1
@@ -64,11 +64,11 @@ class ResidualStream:
             splits = 1
         if splits > 1:
             partials = step.buffer("stream.partials", splits * rows, width, "float32").view(splits, rows, width)
-            K.gemm(a, weight, K.epilogue_f32(partials), splits=splits)
+            K.gemm(a, weight, K.epilogue_f32(partials), splits=splits, packed=packed)
             self.add(Delta(partials, bias))
         else:
             self.flush()
-            K.gemm(a, weight, K.epilogue_residual(self.x, bias))
+            K.gemm(a, weight, K.epilogue_residual(self.x, bias), packed=packed)
 
     def flush(self):
         """Adds what is pending without normalising anything."""
@@ -163,6 +163,16 @@ class Block:
 @functools.lru_cache(maxsize=None)
 def compute_units(device):
     return torch.cuda.get_device_properties(device).multi_processor_count
+
+
+def packed_for_stream(weight):
+    """A matrix's packed copy for the product that adds to the residual stream in decode steps
+    (laid out for the split of K such steps use)."""
+    chunk = 32 if weight.dtype == torch.bfloat16 else 16
+    splits = 1
+    if weight.dtype == torch.bfloat16 or weight.shape[1] % 4 == 0:
+        splits = split_count(K.PackedWeight.ROWS, weight.shape[0], weight.shape[1], compute_units(weight.device), chunk)
+    return K.PackedWeight(weight, splits)
 
 
 def split_count(rows, columns, k, units=256, chunk=32):

@@ -13,7 +13,7 @@ act(0) = 0 in the padded columns, which meet zero columns of the down projection
 import torch
 
 from ..kernels import library as K
-from .base import FeedForward
+from .base import FeedForward, packed_for_stream
 from .registry import register
 
 
@@ -42,8 +42,12 @@ class DenseFeedForward(FeedForward):
             if self.up_bias is not None:
                 self.up_bias = torch.cat([self.up_bias, self.up_bias.new_zeros(extra)]).contiguous()
 
+        # second copies for decode steps, which read the weights and little else
+        self.up_packed = K.PackedWeight(self.up_weight) if self.up_weight.is_cuda else None
+        self.down_packed = packed_for_stream(self.down_weight) if self.down_weight.is_cuda else None
+
     def forward(self, h, step, stream):
         tokens = h.shape[0]
         hidden = step.buffer("feed_forward.hidden", tokens, self.padded, step.dtype)
-        K.gemm(h, self.up_weight, K.epilogue_act(hidden, self.activation, self.up_bias))
-        stream.add_product(step, hidden, self.down_weight, self.down_bias)
+        K.gemm(h, self.up_weight, K.epilogue_act(hidden, self.activation, self.up_bias), packed=self.up_packed)
+        stream.add_product(step, hidden, self.down_weight, self.down_bias, packed=self.down_packed)

@@ -191,6 +191,31 @@ def test_wide_decode_batches(name, dtype, count):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_decoding_from_packed_weight_copies_changes_no_bit(name, dtype):
+    """Decode steps read second copies of the layers' matrices, packed for the skinny kernel; with
+    the copies switched off the same steps read the plain matrices and give the same bits."""
+    from burn_transformers_amd.kernels import library as K
+    runs = []
+    for enabled in (True, False):
+        K.PackedWeight.enabled = enabled
+        try:
+            engine = engine_for(name, dtype, graphs=False)
+            requests = prompts_for(name, [9, 1, 30, 17, 5], seed=11)
+            slots = [engine.open() for _ in requests]
+            rows = [engine.step(list(zip(slots, requests))).clone()]
+            for _ in range(6):
+                ids = rows[-1].argmax(-1).tolist()
+                rows.append(engine.step([(s, [t]) for s, t in zip(slots, ids)]).clone())
+            runs.append(torch.stack(rows))
+        finally:
+            K.PackedWeight.enabled = True
+    assert torch.equal(runs[0], runs[1])
+    mixer = engine.model.blocks[0].parts["mixer"]
+    assert mixer.qkv_packed is not None and mixer.qkv_packed.for_step(5, 1) is not None     # the copies were in use
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_reused_blocks_do_not_leak(dtype):
     """A slot's blocks are poisoned with NaN after it is closed; the next occupant must not care."""
     engine = engine_for("A", dtype, max_tokens=256)

@@ -167,6 +167,54 @@ def test_skinny_gemm_at_decode_sizes(m, n, k, splits, columns, dtype):
         assert rel_err(out, gelu_tanh(want + bias.cpu().double())) < (2e-6 if dtype == "float32" else 6e-3)
 
 
+@pytest.mark.parametrize("m,n,k,splits", [(1, 100, 136, 1), (8, 4800, 1600, 1), (16, 1600, 1608, 4), (7, 333, 6400, 5),
+                                          (3, 50, 40, 1), (33, 517, 1760, 1), (64, 96, 320, 2)])
+@pytest.mark.parametrize("columns", [8, 12, 20, 32])
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_skinny_gemm_reads_packed_weights(m, n, k, splits, columns, dtype):
+    """The same product from the packed copy of the weights (chunks of K one after the other for
+    each work-group's columns, K and the last group padded): right against float64, and bitwise
+    what the plain layout gives, because only the addresses differ."""
+    dt = DTYPES[dtype]
+    a, w, bias, want = operands(m, n, k, dt, seed=k + columns, lda=k + 8)
+    packed = K.pack_columns(w, columns)
+    chunk = 32 if dtype == "bfloat16" else 16
+    assert packed.shape == ((n + columns - 1) // columns, (k + chunk - 1) // chunk, columns, chunk)
+    plain = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    from_packed = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    K.gemm(a, w, K.epilogue_f32(plain, bias), splits=splits, impl="skinny", variant=columns)
+    K.gemm(a, w, K.epilogue_f32(from_packed, bias), splits=splits, impl="skinny", packed=(packed, columns))
+    assert torch.equal(plain, from_packed)
+    assert rel_err(from_packed.sum(0), want + bias.cpu().double()) < (2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k))
+
+
+def test_packed_weight_is_used_only_where_it_fits():
+    """A PackedWeight is laid out for one column count; steps whose launcher would choose another
+    (another split of K, many rows) read the plain matrix, and so does every other kernel."""
+    gen = torch.Generator().manual_seed(5)
+    w = (torch.randn(1600, 640, generator=gen) / 25).to(torch.bfloat16).to(DEV)
+    packed = K.PackedWeight(w, splits=2)
+    units = torch.cuda.get_device_properties(DEV).multi_processor_count
+    assert packed.columns == K.skinny_columns(8, 1600, 640, 2, torch.bfloat16, units)
+    assert packed.for_step(8, 2) is not None and packed.for_step(8, 2)[1] == packed.columns
+    assert packed.for_step(65, 2) is None
+    other = [s for s in (1, 2, 3, 4, 5) if K.skinny_columns(8, 1600, 640, s, torch.bfloat16, units) != packed.columns]
+    for splits in other:
+        assert packed.for_step(8, splits) is None
+    for m, splits in ((1, 2), (8, 2), (16, 1), (40, 2), (100, 1)):
+        a = (torch.randn(m, 640, generator=gen)).to(torch.bfloat16).to(DEV)
+        with_copy = torch.full((splits, m, 1600), float("nan"), dtype=torch.float32, device=DEV)
+        without = torch.full((splits, m, 1600), float("nan"), dtype=torch.float32, device=DEV)
+        K.gemm(a, w, K.epilogue_f32(with_copy), splits=splits, packed=packed, impl="auto" if splits == 1 else "skinny" if m <= 64 else "tile")
+        K.gemm(a, w, K.epilogue_f32(without), splits=splits, impl="auto" if splits == 1 else "skinny" if m <= 64 else "tile")
+        assert torch.equal(with_copy, without)
+    try:
+        K.PackedWeight.enabled = False
+        assert packed.for_step(8, 2) is None
+    finally:
+        K.PackedWeight.enabled = True
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 100, 136), (8, 6400, 1600), (16, 333, 1608), (9, 517, 64), (13, 4800, 2048),
                                    (3, 48, 1024), (16, 96, 1032)])
 @pytest.mark.parametrize("kind,with_shift", [("layer_norm", True), ("rms_norm", False)])

@@ -335,32 +335,38 @@ def skinny_columns(m, n, k, splits, dtype, units):
 
 
 class PackedWeight:
-    """A second copy of a matrix in the skinny kernel's packed form (``pack_columns``), for the
-    column count the launcher chooses for steps of a few rows with ``splits`` slices of K.  Decode
-    steps read weights and little else, and from the packed copy a product of up to 16 rows takes
-    about a seventh less time (6.9 -> 6.0 us for 4800 x 1600, 7.9 -> 6.5 us for 6400 x 1600 at 8
-    rows); results are bitwise the same.  ``for_step`` hands the copy out where it fits the step."""
+    """Second copies of a matrix in the skinny kernel's packed form (``pack_columns``), one for each
+    column count the launcher chooses for steps of a few rows with the given splits of K (a product
+    that adds to the residual stream runs with a split of K or, behind a folded norm, without).
+    Decode steps read weights and little else, and from a packed copy a product of up to 16 rows
+    takes about a seventh less time (6.9 -> 6.0 us for 4800 x 1600, 7.9 -> 6.5 us for 6400 x 1600
+    at 8 rows); results are bitwise the same.  ``for_step`` hands out the copy that fits a step."""
 
-    ROWS = 8            # the step the copy is laid out for; other small steps choose the same columns almost always
+    ROWS = 8            # the step the copies are laid out for; other small steps choose the same columns almost always
     enabled = True      # tests switch it off to run the plain layout too
 
-    def __init__(self, w, splits=1):
-        self.shape, self.dtype, self.splits = tuple(w.shape), w.dtype, splits
+    def __init__(self, w, splits=(1,)):
+        self.shape, self.dtype = tuple(w.shape), w.dtype
         self.units = torch.cuda.get_device_properties(w.device).multi_processor_count
-        self.columns = skinny_columns(self.ROWS, w.shape[0], w.shape[1], splits, w.dtype, self.units)
-        self.tensor = pack_columns(w, self.columns)
+        self.copies = {}                 # columns per work-group -> packed tensor
+        for count in ((splits,) if isinstance(splits, int) else splits):
+            columns = skinny_columns(self.ROWS, w.shape[0], w.shape[1], count, w.dtype, self.units)
+            if columns not in self.copies:
+                self.copies[columns] = pack_columns(w, columns)
         self._fits = {}
 
     def for_step(self, m, splits):
         """(packed tensor, columns) if a product of ``m`` rows and ``splits`` slices runs on the
-        skinny kernel with this copy's columns, else None (the caller then reads the plain matrix)."""
+        skinny kernel with the columns of one of the copies, else None (the caller then reads the
+        plain matrix)."""
         if not PackedWeight.enabled or m > 64:
             return None
         fits = self._fits.get((m, splits))
         if fits is None:
-            fits = skinny_columns(m, self.shape[0], self.shape[1], splits, self.dtype, self.units) == self.columns
+            columns = skinny_columns(m, self.shape[0], self.shape[1], splits, self.dtype, self.units)
+            fits = (self.copies[columns], columns) if columns in self.copies else False
             self._fits[(m, splits)] = fits
-        return (self.tensor, self.columns) if fits else None
+        return fits or None
 
 
 def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):

@@ -167,12 +167,12 @@ def compute_units(device):
 
 def packed_for_stream(weight):
     """A matrix's packed copy for the product that adds to the residual stream in decode steps
-    (laid out for the split of K such steps use)."""
+    (laid out for the split of K such steps use, and for none)."""
     chunk = 32 if weight.dtype == torch.bfloat16 else 16
     splits = 1
     if weight.dtype == torch.bfloat16 or weight.shape[1] % 4 == 0:
         splits = split_count(K.PackedWeight.ROWS, weight.shape[0], weight.shape[1], compute_units(weight.device), chunk)
-    return K.PackedWeight(weight, splits)
+    return K.PackedWeight(weight, (splits, 1))       # (without a split where the norm behind it is folded)
 
 
 def split_count(rows, columns, k, units=256, chunk=32):

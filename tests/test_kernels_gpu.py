@@ -195,10 +195,14 @@ def test_packed_weight_is_used_only_where_it_fits():
     w = (torch.randn(1600, 640, generator=gen) / 25).to(torch.bfloat16).to(DEV)
     packed = K.PackedWeight(w, splits=2)
     units = torch.cuda.get_device_properties(DEV).multi_processor_count
-    assert packed.columns == K.skinny_columns(8, 1600, 640, 2, torch.bfloat16, units)
-    assert packed.for_step(8, 2) is not None and packed.for_step(8, 2)[1] == packed.columns
+    columns = K.skinny_columns(8, 1600, 640, 2, torch.bfloat16, units)
+    assert list(packed.copies) == [columns]
+    assert packed.for_step(8, 2) is not None and packed.for_step(8, 2)[1] == columns
     assert packed.for_step(65, 2) is None
-    other = [s for s in (1, 2, 3, 4, 5) if K.skinny_columns(8, 1600, 640, s, torch.bfloat16, units) != packed.columns]
+    other = [s for s in (1, 2, 3, 4, 5) if K.skinny_columns(8, 1600, 640, s, torch.bfloat16, units) != columns]
+    both = K.PackedWeight(w, splits=(2, 1))
+    assert set(both.copies) == {columns, K.skinny_columns(8, 1600, 640, 1, torch.bfloat16, units)}
+    assert both.for_step(2, 1) is not None
     for splits in other:
         assert packed.for_step(8, splits) is None
     for m, splits in ((1, 2), (8, 2), (16, 1), (40, 2), (100, 1)):

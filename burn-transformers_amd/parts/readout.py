@@ -15,8 +15,11 @@ class LinearReadout(Readout):
         if tuple(self.weight.shape) != (self.vocab_size, self.width):
             raise ValueError(f"readout: table is {tuple(self.weight.shape)}, expected "
                              f"{(self.vocab_size, self.width)}")
+        # a second copy for steps of few rows, which read the table and little else (the token
+        # embedding looks rows up in the table as it is stored)
+        self.packed = K.PackedWeight(self.weight) if self.weight.is_cuda else None
 
     def logits(self, h, step):
         out = step.buffer("readout.logits", h.shape[0], self.vocab_size, "float32")
-        K.gemm(h, self.weight, K.epilogue_f32(out))
+        K.gemm(h, self.weight, K.epilogue_f32(out), packed=self.packed)
         return out

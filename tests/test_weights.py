@@ -184,3 +184,25 @@ def test_in_memory_tensors_go_through_the_same_check():
     del tensors["ln_f.bias"]
     with pytest.raises(bt.WeightError, match="missing tensors \\(1\\): ln_f.bias"):
         store_from_tensors(tensors, contract, torch.float32, "cpu")
+
+
+def test_packed_layout_of_a_matrix():
+    """pack_columns: group g, chunk c, column j, element e of the packed copy is W[g * columns + j,
+    c * chunk + e], zero beyond the matrix (chunks of 32 bfloat16 or 16 float32 values of K)."""
+    import torch
+    from burn_transformers_amd.kernels.library import pack_columns, skinny_columns
+    for dtype, chunk in ((torch.bfloat16, 32), (torch.float32, 16)):
+        w = torch.arange(50 * 72, dtype=torch.float32).reshape(50, 72).to(dtype)
+        packed = pack_columns(w, 12)
+        assert packed.shape == (5, (72 + chunk - 1) // chunk, 12, chunk) and packed.is_contiguous()
+        for g, c, j, e in ((0, 0, 0, 0), (1, 2, 3, 7), (4, 1, 1, 5), (3, 0, 11, chunk - 1)):
+            row, col = g * 12 + j, c * chunk + e
+            want = w[row, col] if row < 50 and col < 72 else 0
+            assert packed[g, c, j, e] == want
+        assert packed[4, 0, 2:].abs().sum() == 0           # rows 50..59 do not exist
+        assert packed[0, -1, :, 72 % chunk:].abs().sum() == 0 or 72 % chunk == 0
+    # the launcher's rule: the fewest rounds of work-groups over the compute units, then the fewest columns
+    assert skinny_columns(8, 4800, 1600, 1, torch.bfloat16, 256) == 20
+    assert skinny_columns(8, 6400, 1600, 1, torch.bfloat16, 256) == 28
+    assert skinny_columns(8, 1600, 6400, 5, torch.bfloat16, 256) == 32
+    assert skinny_columns(8, 1600, 1600, 1, torch.bfloat16, 256) == 8

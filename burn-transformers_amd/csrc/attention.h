@@ -24,4 +24,7 @@ struct AttnArgs {
   // [n_seqs][q_heads][splits][head_dim + 2], and a second kernel joins them into `out`.
   int splits;
   float* partial;
+  // Decode (bfloat16 MFMA kernels) only: 0, or `out` is chunk-major with that many rows
+  // (activation_offset in common.h); ldo is then not used.
+  int out_rows;
 };

@@ -696,7 +696,8 @@ attention_decode_kernel(AttnArgs a) {
       }
     }
     if (splits == 1) {
-      out[(int64_t)tok * a.ldo + (kv_head * group + j) * HD + channel] = (bf16_t)(den > 0.f ? num / den : 0.f);
+      out[activation_offset<bf16_t>(a.out_rows, a.ldo, tok, (kv_head * group + j) * HD + channel)] =
+          (bf16_t)(den > 0.f ? num / den : 0.f);
     } else {     // this run's share, for attention_join_kernel
       float* mine = a.partial + (((int64_t)seq * a.q_heads + kv_head * group + j) * splits + split) * (HD + 2);
       mine[channel] = num;
@@ -715,7 +716,7 @@ attention_join_kernel(AttnArgs a) {
   const float* runs = a.partial + ((int64_t)seq * a.q_heads + head) * a.splits * (HD + 2);
   float top = -INFINITY;
   for (int s = 0; s < a.splits; ++s) top = fmaxf(top, runs[s * (HD + 2) + HD]);
-  bf16_t* out = static_cast<bf16_t*>(a.out) + (int64_t)seq * a.ldo + head * HD;
+  bf16_t* out = static_cast<bf16_t*>(a.out);
   for (int channel = threadIdx.x; channel < HD; channel += 64) {
     float num = 0.f, den = 0.f;
     if (top != -INFINITY) {
@@ -725,7 +726,7 @@ attention_join_kernel(AttnArgs a) {
         den += runs[s * (HD + 2) + HD + 1] * f;
       }
     }
-    out[channel] = (bf16_t)(den > 0.f ? num / den : 0.f);
+    out[activation_offset<bf16_t>(a.out_rows, a.ldo, seq, head * HD + channel)] = (bf16_t)(den > 0.f ? num / den : 0.f);
   }
 }
 
@@ -745,6 +746,7 @@ static int check_args(const AttnArgs& a, const char* who) {
 BT_EXPORT int bt_head_dim() { return HD; }
 
 BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
+  if (args->out_rows != 0) BT_REFUSE("attention_prefill_bf16: a chunk-major output is written by the bfloat16 decode kernel only");
   if (args->n_tokens <= 0 || args->n_seqs <= 0) return BT_OK;
   int rc = check_args(*args, "attention_prefill_bf16");
   if (rc) return rc;
@@ -798,6 +800,8 @@ BT_EXPORT int bt_attention_decode_bf16(void* stream, const AttnArgs* args) {
     BT_REFUSE("attention_decode_bf16: at most 16 query heads per key/value head, got %d",
               args->q_heads / args->kv.kv_heads);
   if (args->n_tokens != args->n_seqs) BT_REFUSE("attention_decode_bf16: needs exactly one token per sequence");
+  if (args->out_rows != 0 && args->out_rows < args->n_tokens)
+    BT_REFUSE("attention_decode_bf16: a chunk-major output of %d rows for %d tokens", args->out_rows, args->n_tokens);
   const int splits = args->splits > 1 ? args->splits : 1;
   if (splits > 1 && !args->partial) BT_REFUSE("attention_decode_bf16: %d runs of keys need a place for their partial results", splits);
   if (splits > 65535 || args->n_seqs > 65535) BT_REFUSE("attention_decode_bf16: %d sequences in %d runs are too many", args->n_seqs, splits);

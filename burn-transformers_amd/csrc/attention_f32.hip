@@ -348,6 +348,7 @@ attention_f32_join_kernel(AttnArgs a) {
 }
 
 BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
+  if (args->out_rows != 0) BT_REFUSE("attention_f32: a chunk-major output is written by the bfloat16 decode kernel only");
   const AttnArgs& a = *args;
   if (a.n_tokens <= 0 || a.n_seqs <= 0) return BT_OK;
   const int hd = a.kv.head_dim;

@@ -68,6 +68,18 @@ __device__ __forceinline__ int value_offset(int head_dim, int pos, int channel) 
   return ((p >> 2) * head_dim + channel) * 4 + (p & 3);
 }
 
+// Activations of a step of few rows may be kept "chunk-major": the chunks of 64 bytes of K (32
+// bfloat16, 16 float32 columns) one after the other, each holding that chunk of every row,
+// [columns / chunk][rows][chunk].  The lanes of an MFMA operand load (16 rows by 64 bytes) then read
+// one contiguous KiB, where row-major rows lie a whole row apart: reading 64 rows of 1,600
+// columns that way takes a work-group 1 us instead of 5.8.  Element offset of (row, column);
+// `rows` = 0 means row-major with the given pitch.
+template <typename T>
+__host__ __device__ __forceinline__ int64_t activation_offset(int rows, int64_t pitch, int row, int column) {
+  constexpr int CHUNK = 64 / (int)sizeof(T);
+  return rows > 0 ? ((int64_t)(column / CHUNK) * rows + row) * CHUNK + column % CHUNK : (int64_t)row * pitch + column;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -58,7 +58,7 @@ __global__ void add_norm_kernel(float* __restrict__ x, const float* __restrict__
                                 int64_t delta_stride, const float* __restrict__ bias,
                                 const float* __restrict__ gamma, const float* __restrict__ beta,
                                 float eps, int kind, T* __restrict__ out, const int* __restrict__ rows,
-                                int width, int write_back) {
+                                int width, int write_back, int out_rows) {
   extern __shared__ float row_buf[];
   __shared__ float scratch[32];
   int r = blockIdx.x;
@@ -88,11 +88,10 @@ __global__ void add_norm_kernel(float* __restrict__ x, const float* __restrict__
     rstd = 1.0f / sqrtf(total / (float)width + eps);
   }
   if (out == nullptr) return;
-  T* orow = out + (int64_t)r * width;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float y = (row_buf[c] - mean) * rstd * gamma[c];
     if (beta) y += beta[c];
-    orow[c] = from_float<T>(y);
+    out[activation_offset<T>(out_rows, width, r, c)] = from_float<T>(y);
   }
 }
 
@@ -109,7 +108,7 @@ __global__ void __launch_bounds__(256)
 add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int64_t delta_stride,
                     const float* __restrict__ bias, const float* __restrict__ gamma,
                     const float* __restrict__ beta, float eps, int kind, T* __restrict__ out,
-                    const int* __restrict__ rows, int width, int write_back) {
+                    const int* __restrict__ rows, int width, int write_back, int out_rows) {
   __shared__ float scratch[32];
   const int r = blockIdx.x;
   const int t = rows ? rows[r] : r;
@@ -173,7 +172,8 @@ add_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ delta, int6
     if (c >= quads) continue;
     float y[4] = {(v[i].x - mean) * rstd * g[i].x + be[i].x, (v[i].y - mean) * rstd * g[i].y + be[i].y,
                   (v[i].z - mean) * rstd * g[i].z + be[i].z, (v[i].w - mean) * rstd * g[i].w + be[i].w};
-    store4<T>(orow + 4 * c, y, 4, true);
+    if (out_rows == 0) store4<T>(orow + 4 * c, y, 4, true);        // (the same branch for every thread)
+    else store4<T>(out + activation_offset<T>(out_rows, width, r, 4 * c), y, 4, true);
   }
 }
 
@@ -261,10 +261,10 @@ add_norm_rows_kernel(float* __restrict__ x, const float* __restrict__ delta, int
 template <typename T, int VPT>
 static bool launch_add_norm_vec(hipStream_t stream, dim3 grid, float* x, const float* delta, int n_delta,
                                 int64_t delta_stride, const float* bias, const float* gamma, const float* beta,
-                                float eps, int kind, T* out, const int* rows, int width, int write_back) {
+                                float eps, int kind, T* out, const int* rows, int width, int write_back, int out_rows) {
 #define BT_ADD_NORM_VEC(NS)                                                                                  \
   hipLaunchKernelGGL((add_norm_vec_kernel<T, VPT, NS>), grid, dim3(256), 0, stream, x, delta, delta_stride,  \
-                     bias, gamma, beta, eps, kind, out, rows, width, write_back)
+                     bias, gamma, beta, eps, kind, out, rows, width, write_back, out_rows)
   switch (n_delta) {
     case 0: BT_ADD_NORM_VEC(0); return true;
     case 1: BT_ADD_NORM_VEC(1); return true;
@@ -283,13 +283,13 @@ static bool launch_add_norm_vec(hipStream_t stream, dim3 grid, float* x, const f
 template <typename T>
 static void launch_add_norm(hipStream_t stream, float* x, const float* delta, int n_delta, int64_t delta_stride,
                             const float* bias, const float* gamma, const float* beta, float eps, int kind,
-                            T* out, const int* rows, int n_rows, int width, int write_back) {
+                            T* out, const int* rows, int n_rows, int width, int write_back, int out_rows) {
   dim3 grid(n_rows);
   auto aligned = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
   bool vec = width % 4 == 0 && width <= 4096 && delta_stride % 4 == 0 && aligned(x) && aligned(delta) &&
              aligned(bias) && aligned(gamma) && aligned(beta) && aligned(out);
   bool done = false;
-  if (vec && n_rows >= 512) {        // many rows: a wave per row
+  if (vec && n_rows >= 512 && out_rows == 0) {        // many rows: a wave per row (row-major output only)
     dim3 row_grid((n_rows + 3) / 4);
 #define BT_ADD_NORM_ROWS(QPL)                                                                                   \
   hipLaunchKernelGGL((add_norm_rows_kernel<T, QPL>), row_grid, dim3(256), 0, stream, x, delta, n_delta,          \
@@ -301,29 +301,31 @@ static void launch_add_norm(hipStream_t stream, float* x, const float* delta, in
     return;
   }
   if (vec && width <= 1024)
-    done = launch_add_norm_vec<T, 1>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+    done = launch_add_norm_vec<T, 1>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back, out_rows);
   else if (vec && width <= 2048)
-    done = launch_add_norm_vec<T, 2>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+    done = launch_add_norm_vec<T, 2>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back, out_rows);
   else if (vec)
-    done = launch_add_norm_vec<T, 4>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+    done = launch_add_norm_vec<T, 4>(stream, grid, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back, out_rows);
   if (!done)
     hipLaunchKernelGGL(add_norm_kernel<T>, grid, dim3(256), (size_t)width * sizeof(float), stream, x, delta,
-                       n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back);
+                       n_delta, delta_stride, bias, gamma, beta, eps, kind, out, rows, width, write_back, out_rows);
 }
 
 BT_EXPORT int bt_add_norm(void* stream, int out_dtype, float* x, const float* delta, int n_delta,
                           int64_t delta_stride, const float* bias, const float* gamma,
                           const float* beta, float eps, int kind, void* out, const int* rows,
-                          int n_rows, int width, int write_back) {
+                          int n_rows, int width, int write_back, int out_rows) {
   if (n_rows <= 0) return BT_OK;
+  if (out_rows != 0 && (out == nullptr || out_rows < n_rows))
+    BT_REFUSE("add_norm: a chunk-major output of %d rows for %d rows", out_rows, n_rows);
   if (width <= 0 || width > 15360) BT_REFUSE("add_norm: width %d outside 1..15360 (the row is held in LDS)", width);
   if (kind != 0 && kind != 1) BT_REFUSE("add_norm: unknown norm kind %d", kind);
   if (out_dtype == 0)
     launch_add_norm<float>((hipStream_t)stream, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind,
-                           (float*)out, rows, n_rows, width, write_back);
+                           (float*)out, rows, n_rows, width, write_back, out_rows);
   else
     launch_add_norm<bf16_t>((hipStream_t)stream, x, delta, n_delta, delta_stride, bias, gamma, beta, eps, kind,
-                            (bf16_t*)out, rows, n_rows, width, write_back);
+                            (bf16_t*)out, rows, n_rows, width, write_back, out_rows);
   return bt_check_launch("add_norm");
 }
 
@@ -490,6 +492,7 @@ int bt_check_attention(const AttnArgs& a, const char* who) {
 }
 
 BT_EXPORT int bt_attention_plain(void* stream, int dtype, const AttnArgs* args) {
+  if (args->out_rows != 0) BT_REFUSE("attention_plain: a chunk-major output is written by the bfloat16 decode kernel only");
   if (args->n_tokens <= 0) return BT_OK;
   int rc = bt_check_attention(*args, "attention_plain");
   if (rc) return rc;

@@ -32,6 +32,7 @@ struct Epilogue {
   const int* tok_seq;    // [M] index of the token's sequence in the step
   const int* tok_pos;    // [M] position of the token in its sequence
   KvView kv;
+  int out_rows;          // EPI_STORE, EPI_ACT: 0, or `out` is chunk-major with that many rows (activation_offset)
 };
 
 // 32-bit activations.  The float32 path (T = float) uses the library's tanhf / erff; the
@@ -136,11 +137,11 @@ __device__ __forceinline__ void epilogue4_prefetched(const Epilogue& e, int N, i
   for (int i = 0; i < 4; ++i) v[i] = acc[i] + p.add[i];
   bool aligned = (e.ldo & 3) == 0;
   if (e.mode == EPI_STORE) {
-    store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
   } else if (e.mode == EPI_ACT) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = activate<T>(v[i], e.act);
-    store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
   } else if (e.mode == EPI_F32) {
     store4<float>(static_cast<float*>(e.out) + (int64_t)split * e.split_stride + (int64_t)m * e.ldo + n0,
                   v, count, aligned);
@@ -181,11 +182,11 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int N, int m, int n
   }
   bool aligned = (e.ldo & 3) == 0;
   if (e.mode == EPI_STORE) {
-    store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
   } else if (e.mode == EPI_ACT) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = activate<T>(v[i], e.act);
-    store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
+    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
   } else if (e.mode == EPI_F32) {
     store4<float>(static_cast<float*>(e.out) + (int64_t)split * e.split_stride + (int64_t)m * e.ldo + n0,
                   v, count, aligned);

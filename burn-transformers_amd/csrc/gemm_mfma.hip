@@ -498,7 +498,7 @@ __device__ float bt_norm_zeros[4] = {0.f, 0.f, 0.f, 0.f};
 template <typename T, int MT, int NT, int U, int WAVES, int QPL = 0>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W, int M, int N,
-                   int K, Epilogue epi, int tile_columns, NormOperand norm, int packed) {
+                   int K, Epilogue epi, int tile_columns, NormOperand norm, int packed, int a_rows) {
   constexpr int ELEMS = Mma<T>::ELEMS;      // K values in a lane's 16-byte load
   constexpr int CHUNK = 4 * ELEMS;          // K values the wave's four K groups cover together
   constexpr bool NORM = QPL > 0;
@@ -531,11 +531,15 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
     w_row[nt] = packed ? W + ((int64_t)blockIdx.x * ((K + CHUNK - 1) / CHUNK) * tile_columns + (n - n_base)) * CHUNK
                        : W + (int64_t)n * K;
   }
+  // a_rows > 0: the activations are chunk-major (activation_offset in common.h) with that many
+  // rows: the 64 lanes of an operand load then read one contiguous KiB
+  const int a_chunk_pitch = a_rows > 0 ? a_rows * CHUNK : CHUNK;      // elements from one chunk of a row to its next
   const T* a_row[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     int m = mt * 16 + i16;
-    a_row[mt] = A + (int64_t)(m < M ? m : M - 1) * lda;
+    m = m < M ? m : M - 1;
+    a_row[mt] = a_rows > 0 ? A + (int64_t)m * CHUNK : A + (int64_t)m * lda;
   }
   // A batch is two phases.  First every load of the batch is issued: a chunk beyond K is
   // skipped by a scalar branch, a group beyond K (a multiple of the group) inside the last chunk
@@ -566,8 +570,10 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wv[u][nt] = *reinterpret_cast<const int4v*>(w_row[nt] + wc);
         if constexpr (!NORM) {
+          // (kc is a multiple of ELEMS inside one chunk: chunk kc / CHUNK, offset kc % CHUNK)
+          int ac = a_rows > 0 ? (kc / CHUNK) * a_chunk_pitch + kc % CHUNK : kc;
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + kc);
+          for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + ac);
         }
       }
     }
@@ -696,6 +702,8 @@ static int check_operands(const char* who, int elems, const void* A, int64_t lda
   if (e.mode < 0 || e.mode > 4 || e.out == nullptr) BT_REFUSE("%s: bad epilogue", who);
   if (splits < 1 || (splits > 1 && e.mode != EPI_F32))
     BT_REFUSE("%s: K can be split %d ways only into 32-bit partial sums", who, splits);
+  if (e.out_rows != 0 && ((e.mode != EPI_STORE && e.mode != EPI_ACT) || e.out_rows < M))
+    BT_REFUSE("%s: a chunk-major output of %d rows for %d rows (stored or activated results only)", who, e.out_rows, M);
   if (e.mode == EPI_QKV) {
     if (e.kv.head_dim <= 0 || e.kv.head_dim % 16 != 0)
       BT_REFUSE("%s: head size %d must be a multiple of 16", who, e.kv.head_dim);
@@ -768,11 +776,11 @@ BT_EXPORT int bt_gemm_tile(void* stream, int dtype, const void* A, int64_t lda, 
 
 template <typename T>
 static void launch_skinny(hipStream_t s, const T* a, int64_t lda, const T* w, int M, int N, int K, const Epilogue& epi,
-                          int splits, int columns, int packed) {
+                          int splits, int columns, int packed, int a_rows) {
   dim3 grid((N + columns - 1) / columns, splits), block(512);
   const NormOperand none = {};
 #define LAUNCH_SKINNY(MT, NT, U) \
-  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns, none, packed)
+  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns, none, packed, a_rows)
   if (M <= 16) {
     if (columns <= 16) LAUNCH_SKINNY(1, 1, 8); else LAUNCH_SKINNY(1, 2, 8);
   } else if (M <= 32) {
@@ -798,7 +806,7 @@ static int launch_skinny_norm(hipStream_t s, const NormOperand& norm, const bf16
       if (err != hipSuccess) BT_REFUSE("gemm_skinny: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));   \
       granted = lds;                                                                                           \
     }                                                                                                          \
-    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)nullptr, (int64_t)0, w, M, N, K, epi, columns, norm, packed); \
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)nullptr, (int64_t)0, w, M, N, K, epi, columns, norm, packed, 0); \
   } while (0)
   if (K <= 1024) {
     if (columns <= 16) LAUNCH_NORM(1, 4); else LAUNCH_NORM(2, 4);
@@ -810,14 +818,19 @@ static int launch_skinny_norm(hipStream_t s, const NormOperand& norm, const bf16
 }
 
 // norm: null, or the activations are the normalised rows it describes (then A and lda are ignored)
+// a_rows: 0, or A is chunk-major with that many rows (activation_offset in common.h; lda is not used).
 // packed_columns: 0, or W is the packed form of the matrix for that many columns per work-group (see
 // the kernel), which then is the number of columns a work-group takes.
 BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda, const void* W, int M, int N, int K,
-                             const Epilogue* epi, int splits, int variant, const NormOperand* norm, int packed_columns) {
+                             const Epilogue* epi, int splits, int variant, const NormOperand* norm, int packed_columns,
+                             int a_rows) {
   if (M <= 0) return BT_OK;
   if (M > 64) BT_REFUSE("gemm_skinny: %d rows, at most 64", M);
   if (dtype != 0 && dtype != 1) BT_REFUSE("gemm_skinny: element type %d is neither float nor bfloat16", dtype);
   const int elems = dtype == 0 ? 4 : 8;
+  if (a_rows != 0 && (norm != nullptr || a_rows < M))
+    BT_REFUSE("gemm_skinny: chunk-major activations of %d rows for a product of %d rows%s", a_rows, M,
+              norm != nullptr ? " that normalises its rows itself" : "");
   if (norm != nullptr) {
     if (dtype != 1 || M > 16 || K > 2048)
       BT_REFUSE("gemm_skinny: the fused norm takes bfloat16 weights, up to 16 rows and K up to 2048 (got %d rows, K %d)", M, K);
@@ -827,6 +840,7 @@ BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda
     A = W;            // (only its alignment is looked at below)
     lda = K;
   }
+  if (a_rows != 0) lda = K;          // (chunk-major rows have no pitch; K itself is checked)
   int rc = check_operands("gemm_skinny", elems, A, lda, W, M, N, K, *epi, splits);
   if (rc) return rc;
   // 8 to 32 columns per work-group in steps of four (one or two column blocks of the kernel),
@@ -863,9 +877,9 @@ BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda
     rc = launch_skinny_norm((hipStream_t)stream, *norm, (const bf16_t*)W, M, N, K, *epi, splits, columns, packed);
     if (rc) return rc;
   } else if (dtype == 0) {
-    launch_skinny<float>((hipStream_t)stream, (const float*)A, lda, (const float*)W, M, N, K, *epi, splits, columns, packed);
+    launch_skinny<float>((hipStream_t)stream, (const float*)A, lda, (const float*)W, M, N, K, *epi, splits, columns, packed, a_rows);
   } else {
-    launch_skinny<bf16_t>((hipStream_t)stream, (const bf16_t*)A, lda, (const bf16_t*)W, M, N, K, *epi, splits, columns, packed);
+    launch_skinny<bf16_t>((hipStream_t)stream, (const bf16_t*)A, lda, (const bf16_t*)W, M, N, K, *epi, splits, columns, packed, a_rows);
   }
   return bt_check_launch("gemm_skinny");
 }

@@ -39,7 +39,7 @@ class KvView(ctypes.Structure):
 class Epilogue(ctypes.Structure):
     _fields_ = [("mode", _c_int), ("act", _c_int), ("bias", _c_ptr), ("out", _c_ptr),
                 ("ldo", _c_i64), ("split_stride", _c_i64), ("n_q", _c_int), ("n_kv", _c_int),
-                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView)]
+                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView), ("out_rows", _c_int)]
 
 
 class AttnArgs(ctypes.Structure):
@@ -47,12 +47,57 @@ class AttnArgs(ctypes.Structure):
                 ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("seq_off", _c_ptr), ("seq_start", _c_ptr),
                 ("kv", KvView), ("q_heads", _c_int), ("n_tokens", _c_int), ("n_seqs", _c_int),
                 ("max_count", _c_int), ("window", _c_int), ("scale", _c_float), ("splits", _c_int),
-                ("partial", _c_ptr)]
+                ("partial", _c_ptr), ("out_rows", _c_int)]
 
 
 class NormOperand(ctypes.Structure):
     _fields_ = [("x", _c_ptr), ("ldx", _c_i64), ("gamma", _c_ptr), ("beta", _c_ptr), ("eps", _c_float),
                 ("kind", _c_int)]
+
+
+class Chunked:
+    """Activations of a step of few rows kept chunk-major: the chunks of 64 bytes of the columns (32
+    bfloat16 or 16 float32 values) one after the other, each with that chunk of every row,
+    [columns / chunk][rows][chunk] (``activation_offset`` in csrc/common.h).  The skinny product
+    reads its rows sixteen at a time, 64 bytes of each: from row-major rows those lie a whole row
+    apart, from this layout they are one contiguous KiB (for 64 rows of 1,600 columns a work-group
+    needs 1 us instead of 5.8 us to read them).  Written by the norm kernel, the decode attention
+    kernel and the products' store / activation epilogues; read by the skinny product only.  It
+    stands where a tensor [rows, columns] would; whoever only hands it on to ``gemm``, ``add_norm``
+    or ``attention_args`` needs to know nothing of it."""
+
+    # Steps of 17 to 64 rows use it.  Up to 16 rows it loses: the norm's rows are written by one
+    # work-group each, and two rows share every 128-byte line of a chunk (measured at 8 rows: the
+    # norm 4.0 -> 4.6 us, the products behind it 6.3 -> 6.8 us; at 64 rows a step gains 5 %).
+    MIN_ROWS, MAX_ROWS = 17, 64
+    enabled = True        # tests switch it off to compare with row-major activations
+
+    @classmethod
+    def wanted(cls, rows):
+        return cls.enabled and cls.MIN_ROWS <= rows <= cls.MAX_ROWS
+
+    def __init__(self, data, rows, columns):
+        self.data, self.shape = data, (rows, columns)
+        self.dtype, self.device = data.dtype, data.device
+
+    @classmethod
+    def take(cls, step, key, rows, columns, dtype):
+        """A chunk-major buffer [rows, columns] from the step's workspace."""
+        chunk = 64 // (2 if dtype == torch.bfloat16 else 4)
+        padded = (columns + chunk - 1) // chunk * chunk
+        return cls(step.buffer(key + ".chunked", rows, padded, dtype), rows, columns)
+
+    def to_rows(self):
+        """The same values as a row-major tensor (tests)."""
+        rows, columns = self.shape
+        chunk = 64 // self.data.element_size()
+        return self.data.view(-1, rows, chunk).permute(1, 0, 2).reshape(rows, -1)[:, :columns]
+
+    def stride(self, dim):
+        return self.shape[1] if dim == 0 else 1
+
+    def data_ptr(self):
+        return self.data.data_ptr()
 
 
 class Normalized:
@@ -80,11 +125,11 @@ _P = ctypes.POINTER
 _SIGNATURES = {
     "bt_embed": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int],
     "bt_add_norm": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_int,
-                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int],
+                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int],
     "bt_gemm_plain": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue)],
     "bt_gemm_tile": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue), _c_int, _c_int],
     "bt_gemm_skinny": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue), _c_int, _c_int,
-                       _P(NormOperand), _c_int],
+                       _P(NormOperand), _c_int, _c_int],
     "bt_gemm_library_bf16": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue)],
     "bt_attention_plain": [_c_ptr, _c_int, _P(AttnArgs)],
     "bt_attention_f32": [_c_ptr, _P(AttnArgs)],
@@ -243,18 +288,25 @@ _library_refused = set()     # (rows, columns, k, epilogue mode, bias?) the libr
 
 
 def _library_takes(epilogue):
+    if epilogue.out_rows:            # chunk-major results are written by this package's kernels only
+        return False
     return epilogue.mode in (EPI_STORE, EPI_RESIDUAL, EPI_F32) or (epilogue.mode == EPI_ACT and epilogue.act == 0)
 
 
 # --- epilogues -------------------------------------------------------------------------------
 
+def _out_rows(out):
+    return out.shape[0] if isinstance(out, Chunked) else 0
+
+
 def epilogue_store(out, bias=None):
-    return Epilogue(mode=EPI_STORE, bias=_ptr(bias), out=out.data_ptr(), ldo=out.stride(0))
+    """``out`` [M, N] in the products' dtype, or a :class:`Chunked` of that shape."""
+    return Epilogue(mode=EPI_STORE, bias=_ptr(bias), out=out.data_ptr(), ldo=out.stride(0), out_rows=_out_rows(out))
 
 
 def epilogue_act(out, activation, bias=None):
     return Epilogue(mode=EPI_ACT, act=ACTIVATIONS[activation], bias=_ptr(bias), out=out.data_ptr(),
-                    ldo=out.stride(0))
+                    ldo=out.stride(0), out_rows=_out_rows(out))
 
 
 def epilogue_f32(out, bias=None):
@@ -287,7 +339,7 @@ def embed(ids, positions, table, position_table, out):
 def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None, rows=None,
              write_back=True):
     """x[t] += sum(delta[:, t]) + bias (kept when ``write_back``); out[r] = norm(x[t]) * gamma + beta
-    with t = rows[r] if rows is given else r.  ``out`` may be None (only the add)."""
+    with t = rows[r] if rows is given else r.  ``out`` may be None (only the add) or a :class:`Chunked`."""
     lib = _module("core")
     width = x.shape[1]
     if delta is None:
@@ -303,8 +355,8 @@ def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None,
     _check(lib, lib.bt_add_norm(
         _stream(), out_dtype, x.data_ptr(), _ptr(delta), n_delta,
         stride, _ptr(bias), _ptr(gamma), _ptr(beta), eps,
-        NORM_KINDS[kind], _ptr(out), _ptr(rows), n_rows, width,
-        1 if write_back else 0))
+        NORM_KINDS[kind], out.data_ptr() if out is not None else None, _ptr(rows), n_rows, width,
+        1 if write_back else 0, _out_rows(out)))
 
 
 def pack_columns(w, columns):
@@ -385,6 +437,12 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
     n = w.shape[0]
     if isinstance(packed, PackedWeight):
         packed = packed.for_step(m, splits) if variant == 0 and impl in ("auto", "skinny") else None
+    a_rows = 0
+    if isinstance(a, Chunked):          # read by the skinny product only
+        if impl not in ("auto", "skinny") or m > Chunked.MAX_ROWS or w.shape[1] != k or not w.is_contiguous() or a.dtype != w.dtype:
+            raise KernelError(f"gemm: chunk-major activations [{m},{k}] {a.dtype} go to the skinny kernel "
+                              f"(up to {Chunked.MAX_ROWS} rows) with weights [{n},{k}] of the same type")
+        impl, a_rows = "skinny", m
     if isinstance(a, Normalized):
         if w.shape[1] != k or not w.is_contiguous() or w.dtype != torch.bfloat16 or impl not in ("auto", "skinny"):
             raise KernelError(f"gemm: rows to be normalised [{m},{k}] go with bfloat16 weights [{n},{k}] on the skinny kernel only")
@@ -393,7 +451,7 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
         lib = _module("gemm_mfma")
         weights, columns = (packed[0].data_ptr(), packed[1]) if packed is not None else (w.data_ptr(), 0)
         _check(lib, lib.bt_gemm_skinny(_stream(), BFLOAT16, None, 0, weights, m, n, k, epilogue, splits,
-                                       variant, operand, columns))
+                                       variant, operand, columns, 0))
         return
     if w.shape[1] != k or a.stride(1) != 1 or not w.is_contiguous() or a.dtype != w.dtype:
         raise KernelError(f"gemm: operands [{m},{k}] {a.dtype} and [{n},{w.shape[1]}] {w.dtype} do not fit")
@@ -428,8 +486,8 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
         _check(lib, lib.bt_gemm_plain(_stream(), dtype, *args))
         return
     if impl == "library":
-        if dtype != BFLOAT16:
-            raise KernelError("gemm: the library product takes bfloat16 only")
+        if dtype != BFLOAT16 or epilogue.out_rows:
+            raise KernelError("gemm: the library product takes bfloat16 only and writes row-major results")
         lib = _library_state["lib"] or library_products()
         if lib is None:
             raise KernelError("gemm: the vendor's GEMM library is not available")
@@ -443,13 +501,14 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
     else:
         if packed is not None:          # (only here: the other kernels read the plain matrix)
             args = (a.data_ptr(), a.stride(0), packed[0].data_ptr(), m, n, k, epilogue)
-        _check(lib, lib.bt_gemm_skinny(_stream(), dtype, *args, splits, variant, None, packed[1] if packed is not None else 0))
+        _check(lib, lib.bt_gemm_skinny(_stream(), dtype, *args, splits, variant, None, packed[1] if packed is not None else 0, a_rows))
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
                    scale, window=0, partial=None):
     """``partial``: float32 [n_seqs * q_heads * runs, head_dim + 2] for a decode step whose keys are
-    cut into runs that separate work-groups take (long contexts in small batches)."""
+    cut into runs that separate work-groups take (long contexts in small batches).  ``out`` may be a
+    :class:`Chunked` for the bfloat16 decode kernels."""
     splits = 1
     if partial is not None:
         splits = partial.shape[0] // (n_seqs * q_heads)
@@ -458,7 +517,7 @@ def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_head
             raise KernelError(f"attention: partial results of shape {tuple(partial.shape)} do not fit "
                               f"{n_seqs} sequences of {q_heads} heads of {kv_view.head_dim}")
     return AttnArgs(splits=splits, partial=partial.data_ptr() if partial is not None and splits > 1 else None,
-                    q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0),
+                    q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0), out_rows=_out_rows(out),
                     tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), seq_off=seq_off.data_ptr(),
                     seq_start=seq_start.data_ptr(), kv=kv_view, q_heads=q_heads, n_tokens=q.shape[0],
                     n_seqs=n_seqs, max_count=max_count, window=window or 0, scale=scale)

@@ -97,7 +97,11 @@ class CausalSelfAttention(Mixer):
             q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
             bias = self.qkv_bias[:self.n_q] if self.qkv_bias is not None else None
             K.gemm(h, self.qkv_weight[:self.n_q], K.epilogue_store(q, bias))
-        mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
+        if step.decode and step.dtype_is_bf16 and K.Chunked.wanted(tokens) \
+                and self.head_dim <= 128 and self.heads // self.kv_heads <= 16:
+            mixed = K.Chunked.take(step, "attention.mixed", tokens, self.n_q, step.dtype)    # the layout the next product reads fastest
+        else:
+            mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
         partial, runs = None, self.decode_runs(step, h.device)
         if runs > 1:
             partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")

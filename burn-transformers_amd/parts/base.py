@@ -99,7 +99,10 @@ class Part:
 
 class Norm(Part):
     def apply(self, stream, step, rows=None):
-        """Normalised rows as a tensor [rows, width] in the step's dtype."""
+        """Normalised rows as a tensor [rows, width] in the step's dtype.  A norm may take a fourth
+        argument ``chunked``: when the block sets it, the part that follows only hands the rows to
+        ``kernels.library.gemm`` (``takes_deferred_norm``), and the norm may return them as a
+        ``kernels.library.Chunked``, the layout the product of a small step reads fastest."""
         raise NotImplementedError
 
     def deferred(self, stream, step):

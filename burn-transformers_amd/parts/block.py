@@ -31,7 +31,7 @@ class PreNormBlock(Block):
         fold_mixer = mixer.takes_deferred_norm and rows <= MIXER_FOLD_ROWS and _can_defer(mixer_norm, step, rows)
         h = mixer_norm.deferred(stream, step) if fold_mixer else None
         if h is None:
-            h = mixer_norm.apply(stream, step)
+            h = _apply(mixer_norm, stream, step, mixer.takes_deferred_norm)
         stream.in_place = fold_ff
         delta = mixer.forward(h, step, memory, stream)
         stream.in_place = False
@@ -39,12 +39,30 @@ class PreNormBlock(Block):
             stream.add(delta)
         h = ff_norm.deferred(stream, step) if fold_ff else None
         if h is None:
-            h = ff_norm.apply(stream, step)
+            h = _apply(ff_norm, stream, step, ff.takes_deferred_norm)
         stream.in_place = fold_mixer          # for the next layer's first norm (or the final one, which does not mind)
         delta = ff.forward(h, step, stream)
         stream.in_place = False
         if delta is not None:
             stream.add(delta)
+
+
+def _apply(norm, stream, step, only_multiplied):
+    """The normalised rows; in a decode step, for a part that only hands them to ``gemm``, in the
+    chunk-major layout if the norm offers it."""
+    if only_multiplied and step.decode and "chunked" in _parameters(type(norm)):
+        return norm.apply(stream, step, chunked=True)
+    return norm.apply(stream, step)
+
+
+_signatures = {}
+
+
+def _parameters(norm_class):
+    if norm_class not in _signatures:
+        import inspect
+        _signatures[norm_class] = frozenset(inspect.signature(norm_class.apply).parameters)
+    return _signatures[norm_class]
 
 
 def _can_defer(norm, step, rows):

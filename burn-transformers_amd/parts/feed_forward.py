@@ -48,6 +48,9 @@ class DenseFeedForward(FeedForward):
 
     def forward(self, h, step, stream):
         tokens = h.shape[0]
-        hidden = step.buffer("feed_forward.hidden", tokens, self.padded, step.dtype)
+        if step.decode and K.Chunked.wanted(tokens) and (step.dtype_is_bf16 or self.padded % 4 == 0):
+            hidden = K.Chunked.take(step, "feed_forward.hidden", tokens, self.padded, step.dtype)   # read by the next product only
+        else:
+            hidden = step.buffer("feed_forward.hidden", tokens, self.padded, step.dtype)
         K.gemm(h, self.up_weight, K.epilogue_act(hidden, self.activation, self.up_bias), packed=self.up_packed)
         stream.add_product(step, hidden, self.down_weight, self.down_bias, packed=self.down_packed)

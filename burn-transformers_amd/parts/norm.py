@@ -22,9 +22,12 @@ class _KernelNorm(Norm):
         if tuple(self.weight.shape) != (self.width,):
             raise ValueError(f"{self.KIND}: scale is {tuple(self.weight.shape)}, expected {(self.width,)}")
 
-    def apply(self, stream, step, rows=None):
+    def apply(self, stream, step, rows=None, chunked=False):
         count = rows.numel() if rows is not None else stream.x.shape[0]
-        out = step.buffer("norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)
+        if chunked and rows is None and K.Chunked.wanted(count) and self.width % 4 == 0:
+            out = K.Chunked.take(step, "norm.out", count, self.width, step.dtype)     # for a part that only hands it to `gemm`
+        else:
+            out = step.buffer("norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)
         pending = stream.pending
         K.add_norm(stream.x, out, self.weight, self.bias, self.eps, self.KIND,
                    delta=pending.partials if pending else None, bias=pending.bias if pending else None,

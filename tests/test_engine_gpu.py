@@ -216,6 +216,35 @@ def test_decoding_from_packed_weight_copies_changes_no_bit(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,count", [("A", 17), ("B", 33), ("C", 40), ("B", 64)])
+def test_chunk_major_activations_change_no_bit(name, count, dtype):
+    """In decode steps of up to 64 sequences the activations between the kernels are kept chunk-major
+    (the layout the skinny product reads fastest); with that switched off the same steps give the
+    same bits."""
+    from burn_transformers_amd.kernels import library as K
+    runs = []
+    for enabled in (True, False):
+        K.Chunked.enabled = enabled
+        try:
+            engine = engine_for(name, dtype, max_tokens=64 * count, graphs=False)
+            requests = prompts_for(name, [2 + (5 * i) % 9 for i in range(count)], seed=33)
+            slots = [engine.open() for _ in requests]
+            rows = []
+            for begin in range(0, count, 8):
+                part = range(begin, min(begin + 8, count))
+                rows.append(engine.step([(slots[i], requests[i]) for i in part]).clone())
+            logits = torch.cat(rows)
+            rows = [logits]
+            for _ in range(4):
+                ids = rows[-1].argmax(-1).tolist()
+                rows.append(engine.step([(s, [t]) for s, t in zip(slots, ids)]).clone())
+            runs.append(torch.stack(rows))
+        finally:
+            K.Chunked.enabled = True
+    assert torch.equal(runs[0], runs[1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_reused_blocks_do_not_leak(dtype):
     """A slot's blocks are poisoned with NaN after it is closed; the next occupant must not care."""
     engine = engine_for("A", dtype, max_tokens=256)

@@ -680,3 +680,82 @@ def test_sampling_is_the_inverse_cdf_of_the_tempered_softmax(rows, vocab):
     assert torch.equal(ids, again)
     K.sample(logits.to(DEV), again, logp, temperature=temperature, seed=seed + 1, first_draw=first, draw_rows=draw_rows)
     assert not torch.equal(ids, again)
+
+
+class _Workspace:
+    """Stands in for a step where only its buffers are asked for."""
+
+    def buffer(self, key, rows, cols, dtype):
+        return torch.full((rows, cols), float("nan"), dtype=dtype, device=DEV)
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("m,n,k,splits", [(1, 100, 136, 1), (8, 4800, 1600, 1), (16, 96, 1608, 3), (17, 333, 320, 1),
+                                          (40, 517, 1760, 2), (64, 1600, 6400, 5), (64, 50, 40, 1)])
+def test_chunk_major_activations_through_the_kernels_that_write_and_read_them(dtype, m, n, k, splits):
+    """Activations of a small step in the chunk-major layout ([columns / chunk][rows][chunk], 64-byte
+    chunks): written by the norm kernel and by a product's store and activation epilogues, read by
+    the skinny product; every value is bitwise what the row-major path gives, only addresses differ."""
+    dt = DTYPES[dtype]
+    gen = torch.Generator().manual_seed(m * 1000 + k)
+    x = (torch.randn(m, k, generator=gen) * 2 + 0.3).to(DEV)
+    gamma = (1 + 0.1 * torch.randn(k, generator=gen)).to(DEV)
+    beta = torch.randn(k, generator=gen).to(DEV)
+    w = (torch.randn(n, k, generator=gen) / math.sqrt(k)).to(dt).to(DEV)
+    bias = torch.randn(n, generator=gen).to(DEV)
+    # the norm writes it
+    rows_out = torch.empty(m, k, dtype=dt, device=DEV)
+    K.add_norm(x.clone(), rows_out, gamma, beta, 1e-5, "layer_norm")
+    chunked = K.Chunked.take(_Workspace(), "test", m, k, dt)
+    K.add_norm(x.clone(), chunked, gamma, beta, 1e-5, "layer_norm")
+    assert chunked.shape == (m, k) and torch.equal(chunked.to_rows(), rows_out)
+    # the skinny product reads it, from the plain and from the packed weights
+    plain = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    K.gemm(rows_out, w, K.epilogue_f32(plain, bias), splits=splits, impl="skinny")
+    for packed in (None, K.PackedWeight(w, splits)):
+        got = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+        K.gemm(chunked, w, K.epilogue_f32(got, bias), splits=splits, packed=packed)
+        assert torch.equal(got, plain)
+    assert rel_err(plain.sum(0), rows_out.double().cpu() @ w.double().cpu().t() + bias.double().cpu()) < (
+        2e-6 if dtype == "float32" else 2e-5 * math.sqrt(k))
+    # a product's epilogues write it
+    if splits == 1:
+        for make in (K.epilogue_store, lambda o, b: K.epilogue_act(o, "gelu_tanh", b)):
+            want = torch.full((m, n), float("nan"), dtype=dt, device=DEV)
+            K.gemm(rows_out, w, make(want, bias), impl="skinny")
+            got = K.Chunked.take(_Workspace(), "test", m, n, dt)
+            K.gemm(chunked, w, make(got, bias))
+            assert torch.equal(got.to_rows(), want)
+    # what cannot read or write it says so
+    with pytest.raises(K.KernelError, match="skinny kernel"):
+        K.gemm(chunked, w, K.epilogue_f32(plain), impl="tile")
+    if dtype == "bfloat16":
+        big = torch.zeros(100, k, dtype=dt, device=DEV)
+        with pytest.raises(K.KernelError, match="row-major"):
+            K.gemm(big, w, K.epilogue_store(K.Chunked.take(_Workspace(), "test", 100, n, dt)), impl="library")
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,hd,totals", [(4, 4, 16, [5, 70, 1]), (6, 2, 48, [300, 64, 65, 1000]),
+                                                        (25, 25, 64, [590] * 8), (8, 1, 128, [33, 2000])])
+def test_decode_attention_writes_chunk_major_rows(q_heads, kv_heads, hd, totals):
+    """The bfloat16 decode kernel (and the kernel that joins runs of keys) leaves its rows in the
+    chunk-major layout when asked: the same bits as row-major; the other attention kernels refuse."""
+    dt = torch.bfloat16
+    case = PagedCase(totals, [1] * len(totals), kv_heads, hd, dt, DEV, seed=hd)
+    gen = torch.Generator().manual_seed(hd + 1)
+    q = (torch.randn(len(totals), q_heads * hd, generator=gen) * 0.5).to(dt).to(DEV)
+    for runs in (1, 3):
+        partial = torch.full((len(totals) * q_heads * runs, hd + 2), float("nan"), device=DEV) if runs > 1 else None
+        want = torch.full((len(totals), q_heads * hd), float("nan"), dtype=dt, device=DEV)
+        args = K.attention_args(q, want, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                                q_heads, len(totals), 1, 0.3, 0, partial)
+        K.attention(args, dt, decode=True)
+        got = K.Chunked.take(_Workspace(), "test", len(totals), q_heads * hd, dt)
+        args = K.attention_args(q, got, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                                q_heads, len(totals), 1, 0.3, 0, partial)
+        K.attention(args, dt, decode=True)
+        assert torch.equal(got.to_rows(), want), runs
+    assert rel_err(want, case.reference(q, q_heads, 0.3, 0)) < 1.2e-2
+    for impl, decode in (("mfma", False), ("plain", True)):
+        with pytest.raises(K.KernelError, match="chunk-major"):
+            K.attention(args, dt, decode=decode, impl=impl)

@@ -48,9 +48,9 @@ class PreNormBlock(Block):
 
 
 def _apply(norm, stream, step, only_multiplied):
-    """The normalised rows; in a decode step, for a part that only hands them to ``gemm``, in the
-    chunk-major layout if the norm offers it."""
-    if only_multiplied and step.decode and "chunked" in _parameters(type(norm)):
+    """The normalised rows; for a part that only hands them to ``gemm``, in the chunk-major layout
+    if the norm offers it (the norm decides by the number of rows)."""
+    if only_multiplied and "chunked" in _parameters(type(norm)):
         return norm.apply(stream, step, chunked=True)
     return norm.apply(stream, step)
 

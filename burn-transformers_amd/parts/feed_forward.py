@@ -48,7 +48,7 @@ class DenseFeedForward(FeedForward):
 
     def forward(self, h, step, stream):
         tokens = h.shape[0]
-        if step.decode and K.Chunked.wanted(tokens) and (step.dtype_is_bf16 or self.padded % 4 == 0):
+        if K.Chunked.wanted(tokens) and (step.dtype_is_bf16 or self.padded % 4 == 0):
             hidden = K.Chunked.take(step, "feed_forward.hidden", tokens, self.padded, step.dtype)   # read by the next product only
         else:
             hidden = step.buffer("feed_forward.hidden", tokens, self.padded, step.dtype)

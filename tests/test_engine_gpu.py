@@ -226,7 +226,7 @@ def test_chunk_major_activations_change_no_bit(name, count, dtype):
     for enabled in (True, False):
         K.Chunked.enabled = enabled
         try:
-            engine = engine_for(name, dtype, max_tokens=64 * count, graphs=False)
+            engine = engine_for(name, dtype, max_tokens=64 * (count + 1), graphs=False)
             requests = prompts_for(name, [2 + (5 * i) % 9 for i in range(count)], seed=33)
             slots = [engine.open() for _ in requests]
             rows = []
@@ -238,6 +238,12 @@ def test_chunk_major_activations_change_no_bit(name, count, dtype):
             for _ in range(4):
                 ids = rows[-1].argmax(-1).tolist()
                 rows.append(engine.step([(s, [t]) for s, t in zip(slots, ids)]).clone())
+            # prompts of 17 to 64 tokens: the norms and the feed-forward use the layout there too
+            for length in (17, 40, 64):
+                slot = engine.open()
+                ids = prompts_for(name, [length], seed=length)[0]
+                rows.append(engine.step([(slot, ids)], want=[[0, length - 1]]).sum(0, keepdim=True).expand(count, -1).clone())
+                engine.close(slot)
             runs.append(torch.stack(rows))
         finally:
             K.Chunked.enabled = True

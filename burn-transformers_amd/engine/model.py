@@ -9,6 +9,7 @@ from ..config.base import read_config_json
 from ..config.registry import resolve_family
 from ..kernels import library as K
 from ..parts import Memory, lookup
+from ..parts.base import offers_chunked
 from ..weights.loader import compute_dtype, load_checkpoint, store_from_tensors
 
 
@@ -78,7 +79,10 @@ class CausalLM:
                 self.blocks[entry.layer].forward(stream, step, memory)
             if not readout:
                 return None
-            hidden = self.final_norm.apply(stream, step, rows=step.sel_rows)
+            if self.readout.takes_deferred_norm and offers_chunked(self.final_norm):
+                hidden = self.final_norm.apply(stream, step, rows=step.sel_rows, chunked=True)
+            else:
+                hidden = self.final_norm.apply(stream, step, rows=step.sel_rows)
             return self.readout.logits(hidden, step)
 
 

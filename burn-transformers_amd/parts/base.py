@@ -112,6 +112,18 @@ class Norm(Part):
         return None
 
 
+_chunked_norms = {}
+
+
+def offers_chunked(norm):
+    """Whether a norm's ``apply`` takes the ``chunked`` argument (see :class:`Norm`)."""
+    kind = type(norm)
+    if kind not in _chunked_norms:
+        import inspect
+        _chunked_norms[kind] = "chunked" in inspect.signature(kind.apply).parameters
+    return _chunked_norms[kind]
+
+
 class Mixer(Part):
     # True for a mixer that hands ``h`` to ``kernels.library.gemm`` and looks at nothing but its
     # shape (see FeedForward.takes_deferred_norm)
@@ -151,6 +163,9 @@ class Embedding(Part):
 
 
 class Readout(Part):
+    # True for a readout that hands ``h`` to ``kernels.library.gemm`` and looks at nothing but its shape
+    takes_deferred_norm = False
+
     def logits(self, h, step):
         raise NotImplementedError
 

@@ -5,7 +5,7 @@ pre_norm: y = x + mixer(norm(x)); z = y + feed_forward(norm(y))
 returns it as a Delta, which stays pending until the next norm reads the stream.
 """
 
-from .base import Block
+from .base import Block, offers_chunked
 from .registry import register
 
 # Most rows of a step whose first norm is folded too.  Measured at GPT-2 XL sizes, ms a decode step
@@ -50,19 +50,9 @@ class PreNormBlock(Block):
 def _apply(norm, stream, step, only_multiplied):
     """The normalised rows; for a part that only hands them to ``gemm``, in the chunk-major layout
     if the norm offers it (the norm decides by the number of rows)."""
-    if only_multiplied and "chunked" in _parameters(type(norm)):
+    if only_multiplied and offers_chunked(norm):
         return norm.apply(stream, step, chunked=True)
     return norm.apply(stream, step)
-
-
-_signatures = {}
-
-
-def _parameters(norm_class):
-    if norm_class not in _signatures:
-        import inspect
-        _signatures[norm_class] = frozenset(inspect.signature(norm_class.apply).parameters)
-    return _signatures[norm_class]
 
 
 def _can_defer(norm, step, rows):

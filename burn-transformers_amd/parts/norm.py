@@ -24,8 +24,8 @@ class _KernelNorm(Norm):
 
     def apply(self, stream, step, rows=None, chunked=False):
         count = rows.numel() if rows is not None else stream.x.shape[0]
-        if chunked and rows is None and K.Chunked.wanted(count) and self.width % 4 == 0:
-            out = K.Chunked.take(step, "norm.out", count, self.width, step.dtype)     # for a part that only hands it to `gemm`
+        if chunked and K.Chunked.wanted(count) and self.width % 4 == 0:
+            out = K.Chunked.take(step, "norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)     # for a part that only hands it to `gemm`
         else:
             out = step.buffer("norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)
         pending = stream.pending

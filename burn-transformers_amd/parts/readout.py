@@ -8,6 +8,8 @@ from .registry import register
 
 @register("readout", "linear_readout")
 class LinearReadout(Readout):
+    takes_deferred_norm = True       # the rows are only handed to ``gemm``: the final norm may leave them chunk-major
+
     def __init__(self, params, tensors):
         super().__init__(params, tensors)
         self.width, self.vocab_size = params["width"], params["vocab_size"]

@@ -172,7 +172,7 @@ __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, in
 // Start of the (block, kv head) plane that holds position kb of a sequence.
 __device__ __forceinline__ int64_t tile_plane(const AttnArgs& a, int seq, int kv_head, int kb) {
   int block = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + kb / BT_KV_BLOCK];
-  return ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
+  return kv_plane(a.kv, block, kv_head);
 }
 
 #ifndef PREFILL_NQ
@@ -646,7 +646,7 @@ attention_decode_kernel(AttnArgs a) {
   // plane of the tile at kb: from the blocks fetched early where they apply, else from the table
   auto plane_of = [&](int kb, int j) {
     int block = (early && j < 2) ? (j == 0 ? early_block0 : early_block1) : block_row[kb / BT_KV_BLOCK];
-    return ((int64_t)block * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * HD);
+    return kv_plane(a.kv, block, kv_head);
   };
   const float c = a.scale * LOG2_E;
   auto fetch = [&](TileOperands& into, int kb, int j) {

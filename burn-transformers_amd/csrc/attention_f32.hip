@@ -70,7 +70,7 @@ attention_f32_kernel(AttnArgs a) {
   floatx4 kreg[LOADS], vreg[LOADS];
   auto fetch = [&](int block) __attribute__((always_inline)) {
     int physical = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + block];
-    int64_t base = ((int64_t)physical * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * hd);
+    int64_t base = kv_plane(a.kv, physical, kv_head);
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
       int piece = tid + 256 * j;
@@ -237,7 +237,7 @@ attention_f32_decode_kernel(AttnArgs a) {
   for (int j = 0; j < CPT; ++j) acc[j] = 0.f;
   for (int block = first_block + wave; block <= last_block; block += 4) {
     int physical = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + block];
-    int64_t base = ((int64_t)physical * a.kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * hd);
+    int64_t base = kv_plane(a.kv, physical, kv_head);
     // this lane's key: row `lane` of the block
     const float4* krow = reinterpret_cast<const float4*>(keys + base + (int64_t)lane * hd);
     const int quads = hd >> 2;

@@ -40,10 +40,14 @@ __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return (bf16_t)v; }  // round to nearest even
 
-// Geometry of one group of layers in the paged key/value storage.
-//   keys:   [layer][block][kv_head][BT_KV_BLOCK][head_dim]
-//   values: [layer][block][kv_head][BT_KV_BLOCK / 4][head_dim][4]   (four positions interleaved
-//           per channel, so that a lane reads four consecutive positions of one channel at once)
+// Geometry of one group of layers in the paged key/value storage.  A (block, head) *plane* holds
+// the keys (or values) of one head for the 64 positions of one block:
+//   keys:   plane = [BT_KV_BLOCK][head_dim]
+//   values: plane = [BT_KV_BLOCK / 4][head_dim][4]   (four positions interleaved per channel, so
+//           that a lane reads four consecutive positions of one channel at once)
+// The plane of (block, head) starts block * block_stride + head * head_stride elements into the
+// layer: the storage decides which of the two lies closer together (with the heads outermost, the
+// blocks a sequence took one after the other are one contiguous run for each head).
 // `blocks` is the table of the step's sequences: blocks[seq * max_blocks + position / BT_KV_BLOCK].
 struct KvView {
   void* keys;            // base of the layer
@@ -52,11 +56,15 @@ struct KvView {
   int max_blocks;
   int kv_heads;
   int head_dim;
+  int64_t block_stride;  // elements from a block's plane to the next block's, same head
+  int64_t head_stride;   // elements from a head's plane to the next head's, same block
 };
 
+__device__ __forceinline__ int64_t kv_plane(const KvView& kv, int block, int kv_head) {
+  return (int64_t)block * kv.block_stride + (int64_t)kv_head * kv.head_stride;
+}
 __device__ __forceinline__ int64_t kv_block_base(const KvView& kv, int seq, int pos, int kv_head) {
-  int block = kv.blocks[(int64_t)seq * kv.max_blocks + pos / BT_KV_BLOCK];
-  return ((int64_t)block * kv.kv_heads + kv_head) * (int64_t)(BT_KV_BLOCK * kv.head_dim);
+  return kv_plane(kv, kv.blocks[(int64_t)seq * kv.max_blocks + pos / BT_KV_BLOCK], kv_head);
 }
 // Element offset of key (pos, channel) inside its (block, head) plane.
 __device__ __forceinline__ int key_offset(int head_dim, int pos, int channel) {

@@ -121,7 +121,7 @@ __device__ __forceinline__ EpiloguePrefetch epilogue_prefetch(const Epilogue& e,
   const int head = kv_column ? c / e.kv.head_dim : 0;
   const int* blocks = kv_column ? e.kv.blocks : bt_dummy_words;
   int block = blocks[kv_column ? (int64_t)seq * e.kv.max_blocks + pos / BT_KV_BLOCK : 0];
-  p.kv_base = ((int64_t)block * e.kv.kv_heads + head) * (int64_t)(BT_KV_BLOCK * e.kv.head_dim);
+  p.kv_base = kv_plane(e.kv, block, head);
   p.pos = pos;
   return p;
 }

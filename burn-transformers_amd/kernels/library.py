@@ -33,7 +33,8 @@ class KernelError(RuntimeError):
 class KvView(ctypes.Structure):
     """One layer of one group of the paged key/value storage, as the kernels see it."""
     _fields_ = [("keys", _c_ptr), ("values", _c_ptr), ("blocks", _c_ptr),
-                ("max_blocks", _c_int), ("kv_heads", _c_int), ("head_dim", _c_int)]
+                ("max_blocks", _c_int), ("kv_heads", _c_int), ("head_dim", _c_int),
+                ("block_stride", _c_i64), ("head_stride", _c_i64)]
 
 
 class Epilogue(ctypes.Structure):

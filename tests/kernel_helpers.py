@@ -54,7 +54,8 @@ class PagedCase:
 
     def view(self):
         return K.KvView(keys=self.keys.data_ptr(), values=self.values.data_ptr(), blocks=self.table.data_ptr(),
-                        max_blocks=self.max_blocks, kv_heads=self.kv_heads, head_dim=self.head_dim)
+                        max_blocks=self.max_blocks, kv_heads=self.kv_heads, head_dim=self.head_dim,
+                        block_stride=self.kv_heads * BLOCK * self.head_dim, head_stride=BLOCK * self.head_dim)
 
     def read_back(self):
         """Keys and values of every position, through the kv_copy kernel."""

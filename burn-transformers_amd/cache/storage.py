@@ -3,8 +3,8 @@ sequence, and the ledger that says who holds what.
 
 Cache entries (one per layer that keeps keys and values, as the model's schedule numbers them)
 with the same :class:`KVSpec` form a *group* with storage of its own:
-    keys    [entries, blocks, kv_heads, 64, head_dim]
-    values  [entries, blocks, kv_heads, 16, head_dim, 4]      (four positions interleaved)
+    [entries, blocks, kv_heads, 2, 64 * head_dim]: for each block and head the plane of its keys,
+    [64, head_dim], beside the plane of its values, [16, head_dim, 4] (four positions interleaved)
 All groups share one block table per sequence, because a sequence is equally long in all of
 them.  Fixed-size state ([entries, slots, *shape], zeroed when a slot is handed out) lives beside
 it for mixers that carry state instead of, or in addition to, keys and values.
@@ -42,10 +42,11 @@ class KVGroup:
         # the blocks of a prompt are one contiguous run for each head) was measured and lost 3 to 4 %
         # of a decode step at batch 8 and 64, also with the heads' runs skewed by a few blocks: the
         # heads of a sequence are read at the same time and written together, and are then far apart.
-        shape = (entries, n_blocks, spec.kv_heads, BLOCK, spec.head_dim)
-        self.keys = torch.zeros(shape, dtype=dtype, device=device)
-        self.values = torch.zeros(shape, dtype=dtype, device=device)
-        self.head_stride = BLOCK * spec.head_dim
+        # A head's keys lie beside its values: what a decode step's work-group reads of a block is
+        # one run of memory (a per cent at batch 64 against two separate tensors)
+        planes = torch.zeros((entries, n_blocks, spec.kv_heads, 2, BLOCK, spec.head_dim), dtype=dtype, device=device)
+        self.keys, self.values = planes[:, :, :, 0], planes[:, :, :, 1]
+        self.head_stride = 2 * BLOCK * spec.head_dim
         self.block_stride = spec.kv_heads * self.head_stride
 
     def view(self, entry, block_table, max_blocks):

@@ -206,3 +206,32 @@ def test_packed_layout_of_a_matrix():
     assert skinny_columns(8, 6400, 1600, 1, torch.bfloat16, 256) == 28
     assert skinny_columns(8, 1600, 6400, 5, torch.bfloat16, 256) == 32
     assert skinny_columns(8, 1600, 1600, 1, torch.bfloat16, 256) == 8
+
+
+def test_chunk_major_layout_of_activations():
+    """Chunked: element (row, column) lies at ((column // chunk) * rows + row) * chunk + column % chunk
+    with chunks of 64 bytes; ``to_rows`` undoes it; the policy takes steps of 17 to 64 rows."""
+    import torch
+    from burn_transformers_amd.kernels.library import Chunked
+
+    class Workspace:
+        def buffer(self, key, rows, cols, dtype):
+            return torch.zeros(rows, cols, dtype=dtype)
+
+    for dtype, chunk in ((torch.bfloat16, 32), (torch.float32, 16)):
+        rows, columns = 5, 72
+        held = Chunked.take(Workspace(), "test", rows, columns, dtype)
+        assert held.shape == (rows, columns) and held.data.numel() == rows * ((columns + chunk - 1) // chunk * chunk)
+        flat = held.data.view(-1)
+        want = torch.arange(rows * columns, dtype=torch.float32).reshape(rows, columns).to(dtype)
+        for r in range(rows):
+            for c in range(columns):
+                flat[((c // chunk) * rows + r) * chunk + c % chunk] = want[r, c]
+        assert torch.equal(held.to_rows(), want)
+        assert held.stride(0) == columns and held.stride(1) == 1 and held.dtype == dtype
+    assert [Chunked.wanted(n) for n in (1, 16, 17, 64, 65)] == [False, False, True, True, False]
+    Chunked.enabled = False
+    try:
+        assert not Chunked.wanted(32)
+    finally:
+        Chunked.enabled = True

@@ -137,11 +137,13 @@ __device__ __forceinline__ void epilogue4_prefetched(const Epilogue& e, int N, i
   for (int i = 0; i < 4; ++i) v[i] = acc[i] + p.add[i];
   bool aligned = (e.ldo & 3) == 0;
   if (e.mode == EPI_STORE) {
-    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
+    if (e.out_rows == 0) store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);     // (one branch for all threads)
+    else store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, true);
   } else if (e.mode == EPI_ACT) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = activate<T>(v[i], e.act);
-    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
+    if (e.out_rows == 0) store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);     // (one branch for all threads)
+    else store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, true);
   } else if (e.mode == EPI_F32) {
     store4<float>(static_cast<float*>(e.out) + (int64_t)split * e.split_stride + (int64_t)m * e.ldo + n0,
                   v, count, aligned);
@@ -182,11 +184,13 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int N, int m, int n
   }
   bool aligned = (e.ldo & 3) == 0;
   if (e.mode == EPI_STORE) {
-    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
+    if (e.out_rows == 0) store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);     // (one branch for all threads)
+    else store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, true);
   } else if (e.mode == EPI_ACT) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = activate<T>(v[i], e.act);
-    store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, aligned || e.out_rows > 0);
+    if (e.out_rows == 0) store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);     // (one branch for all threads)
+    else store4<T>(static_cast<T*>(e.out) + activation_offset<T>(e.out_rows, e.ldo, m, n0), v, count, true);
   } else if (e.mode == EPI_F32) {
     store4<float>(static_cast<float*>(e.out) + (int64_t)split * e.split_stride + (int64_t)m * e.ldo + n0,
                   v, count, aligned);

@@ -495,7 +495,7 @@ struct NormOperand {
 
 __device__ float bt_norm_zeros[4] = {0.f, 0.f, 0.f, 0.f};
 
-template <typename T, int MT, int NT, int U, int WAVES, int QPL = 0>
+template <typename T, int MT, int NT, int U, int WAVES, int QPL = 0, bool CHUNKED = false>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W, int M, int N,
                    int K, Epilogue epi, int tile_columns, NormOperand norm, int packed, int a_rows) {
@@ -531,15 +531,15 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
     w_row[nt] = packed ? W + ((int64_t)blockIdx.x * ((K + CHUNK - 1) / CHUNK) * tile_columns + (n - n_base)) * CHUNK
                        : W + (int64_t)n * K;
   }
-  // a_rows > 0: the activations are chunk-major (activation_offset in common.h) with that many
-  // rows: the 64 lanes of an operand load then read one contiguous KiB
-  const int a_chunk_pitch = a_rows > 0 ? a_rows * CHUNK : CHUNK;      // elements from one chunk of a row to its next
+  // CHUNKED: the activations are chunk-major (activation_offset in common.h) with a_rows rows: the
+  // 64 lanes of an operand load then read one contiguous KiB.  (A form of the kernel of its own, so
+  // that the row-major form keeps its loads free of anything computed per lane between them.)
+  const int a_chunk_pitch = CHUNKED ? a_rows * CHUNK : CHUNK;      // elements from one chunk of a row to its next
   const T* a_row[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     int m = mt * 16 + i16;
-    m = m < M ? m : M - 1;
-    a_row[mt] = a_rows > 0 ? A + (int64_t)m * CHUNK : A + (int64_t)m * lda;
+    a_row[mt] = CHUNKED ? A + (int64_t)(m < M ? m : M - 1) * CHUNK : A + (int64_t)(m < M ? m : M - 1) * lda;
   }
   // A batch is two phases.  First every load of the batch is issued: a chunk beyond K is
   // skipped by a scalar branch, a group beyond K (a multiple of the group) inside the last chunk
@@ -571,7 +571,7 @@ gemm_skinny_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ W
         for (int nt = 0; nt < NT; ++nt) wv[u][nt] = *reinterpret_cast<const int4v*>(w_row[nt] + wc);
         if constexpr (!NORM) {
           // (kc is a multiple of ELEMS inside one chunk: chunk kc / CHUNK, offset kc % CHUNK)
-          int ac = a_rows > 0 ? (kc / CHUNK) * a_chunk_pitch + kc % CHUNK : kc;
+          int ac = CHUNKED ? (kc / CHUNK) * a_chunk_pitch + kc % CHUNK : kc;
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) av[u][mt] = *reinterpret_cast<const int4v*>(a_row[mt] + ac);
         }
@@ -779,8 +779,15 @@ static void launch_skinny(hipStream_t s, const T* a, int64_t lda, const T* w, in
                           int splits, int columns, int packed, int a_rows) {
   dim3 grid((N + columns - 1) / columns, splits), block(512);
   const NormOperand none = {};
-#define LAUNCH_SKINNY(MT, NT, U) \
-  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns, none, packed, a_rows)
+#define LAUNCH_SKINNY(MT, NT, U)                                                                                   \
+  do {                                                                                                             \
+    if (a_rows > 0)                                                                                                \
+      hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8, 0, true>), grid, block, 0, s, a, lda, w, M, N, K, epi, \
+                         columns, none, packed, a_rows);                                                           \
+    else                                                                                                           \
+      hipLaunchKernelGGL((gemm_skinny_kernel<T, MT, NT, U, 8>), grid, block, 0, s, a, lda, w, M, N, K, epi, columns, \
+                         none, packed, 0);                                                                         \
+  } while (0)
   if (M <= 16) {
     if (columns <= 16) LAUNCH_SKINNY(1, 1, 8); else LAUNCH_SKINNY(1, 2, 8);
   } else if (M <= 32) {

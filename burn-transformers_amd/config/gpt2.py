@@ -89,6 +89,10 @@ class GPT2Config:
             raise ConfigError(FAMILY, "add_cross_attention", "cross-attention blocks are not implemented")
         if not self.tie_word_embeddings:
             raise ConfigError(FAMILY, "tie_word_embeddings", "the readout must be tied to the token embedding")
+        if not self.causal:
+            # the reference's stateless module can run unmasked (src/models/gpt2.rs:141); a cached
+            # step cannot: a token's keys would have to include tokens that are not there yet
+            raise ConfigError(FAMILY, "causal", "only causal attention can run from a cache")
         if self.n_inner is not None and not (0 < self.n_inner <= 2 ** 62):
             raise ConfigError(FAMILY, "n_inner", "must be positive and fit usize")
         for width in (self.vocab_size, self.n_positions, self.intermediate_size, 3):

@@ -383,9 +383,8 @@ int bt_check_epilogue(const Epilogue& e, int N, const char* who) {
   if (e.mode < 0 || e.mode > 4) BT_REFUSE("%s: unknown epilogue mode %d", who, e.mode);
   if (e.out == nullptr) BT_REFUSE("%s: epilogue has no output", who);
   if (e.mode == EPI_QKV) {
-    if (e.kv.head_dim <= 0 || e.kv.head_dim % 16 != 0)
-      BT_REFUSE("%s: head size %d must be a multiple of 16", who, e.kv.head_dim);
-    if (e.n_q % 16 != 0 || e.n_kv != e.kv.kv_heads * e.kv.head_dim || e.n_q + 2 * e.n_kv != N)
+    if (e.kv.head_dim <= 0) BT_REFUSE("%s: head size %d must be positive", who, e.kv.head_dim);
+    if (e.n_q % e.kv.head_dim != 0 || e.n_kv != e.kv.kv_heads * e.kv.head_dim || e.n_q + 2 * e.n_kv != N)
       BT_REFUSE("%s: fused projection of %d columns does not split into %d query and 2 x %d key/value columns",
                 who, N, e.n_q, e.n_kv);
     if (!e.tok_seq || !e.tok_pos || !e.kv.blocks || !e.kv.keys || !e.kv.values)
@@ -481,7 +480,7 @@ attention_plain_kernel(AttnArgs a) {
 
 int bt_check_attention(const AttnArgs& a, const char* who) {
   int hd = a.kv.head_dim;
-  if (hd <= 0 || hd % 16 != 0 || hd > 256) BT_REFUSE("%s: head size %d must be a multiple of 16 up to 256", who, hd);
+  if (hd <= 0 || hd > 256) BT_REFUSE("%s: head size %d outside 1..256 (a work-group holds a query and one channel per thread)", who, hd);
   if (a.kv.kv_heads <= 0 || a.q_heads <= 0 || a.q_heads % a.kv.kv_heads != 0)
     BT_REFUSE("%s: %d query heads cannot share %d key/value heads", who, a.q_heads, a.kv.kv_heads);
   if (a.window < 0) BT_REFUSE("%s: window %d must not be negative", who, a.window);
@@ -609,7 +608,7 @@ BT_EXPORT int bt_kv_copy(void* stream, int dtype, void* k_rows, void* v_rows, in
                          const int* tok_seq, const int* tok_pos, const KvView* kv, int tokens,
                          int to_cache) {
   if (tokens <= 0) return BT_OK;
-  if (kv->head_dim <= 0 || kv->head_dim % 4 != 0) BT_REFUSE("kv_copy: head size %d must be a multiple of 4", kv->head_dim);
+  if (kv->head_dim <= 0) BT_REFUSE("kv_copy: head size %d must be positive", kv->head_dim);
   dim3 grid(tokens), block(256);
   const bool wide = dtype != 0 && to_cache && tokens > 64 && kv->head_dim % 8 == 0 && ld % 8 == 0 &&
                     ((uintptr_t)k_rows & 15) == 0 && ((uintptr_t)v_rows & 15) == 0 && ((uintptr_t)kv->keys & 15) == 0 &&

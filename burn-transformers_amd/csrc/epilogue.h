@@ -200,7 +200,27 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int N, int m, int n
     for (int i = 0; i < 4; ++i)
       if (i < count) v[i] += x[i];
     store4<float>(x, v, count, aligned);
-  } else {  // EPI_QKV: n_q, n_kv and head_dim are multiples of 16, so the four columns share a head
+  } else if ((e.kv.head_dim & 3) != 0) {
+    // EPI_QKV with a head size that four columns do not divide (the plain product only): every
+    // column finds its own place among the queries, keys and values
+    int seq = e.tok_seq[m], pos = e.tok_pos[m];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i >= count) break;
+      int n = n0 + i;
+      if (n < e.n_q) {
+        static_cast<T*>(e.out)[(int64_t)m * e.ldo + n] = from_float<T>(v[i]);
+        continue;
+      }
+      int c = n - e.n_q;
+      bool is_value = c >= e.n_kv;
+      if (is_value) c -= e.n_kv;
+      int head = c / e.kv.head_dim, channel = c % e.kv.head_dim;
+      int64_t base = kv_block_base(e.kv, seq, pos, head);
+      if (!is_value) static_cast<T*>(e.kv.keys)[base + key_offset(e.kv.head_dim, pos, channel)] = from_float<T>(v[i]);
+      else static_cast<T*>(e.kv.values)[base + value_offset(e.kv.head_dim, pos, channel)] = from_float<T>(v[i]);
+    }
+  } else {  // EPI_QKV: head_dim (and with it n_q and n_kv) is a multiple of four, so the four columns share a head
     if (n0 < e.n_q) {
       store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);
     } else {

@@ -34,7 +34,7 @@ _MAX_GRAPHS = 48           # graphs kept; the one that was used longest ago goes
 
 
 class StepError(ValueError):
-    """The step was refused; the cache is as it was."""
+    """The step was refused before anything ran; the cache is as it was."""
 
 
 class Engine:
@@ -45,8 +45,7 @@ class Engine:
                            model.dtype, model.device, max_slots)
         self.pool = BufferPool(self.device)
         # a mixer that plans work on the host per step cannot be replayed from a graph
-        self.use_graphs = graphs and all(getattr(block.parts.get("mixer"), "graph_safe", True)
-                                         for block in model.blocks)
+        self.use_graphs = graphs and all(mixer.graph_safe for block in model.blocks for mixer in block.mixers())
         self._meta = None                  # device int32 buffer of eager steps
         self._pinned = []                  # ring of (pinned int32 tensor, event)
         self._pinned_next = 0
@@ -92,7 +91,10 @@ class Engine:
                 size, low, high = 1, tokens[0], tokens[0]      # a decode step's entry: no array is made for it
                 ids.append(tokens[0])
             else:
-                tokens = np.asarray(tokens, dtype=np.int64).reshape(-1)
+                tokens = np.asarray(tokens)
+                if tokens.size and tokens.dtype.kind not in "iu":
+                    raise StepError(f"token ids of slot {slot} are {tokens.dtype} values, expected integers")
+                tokens = tokens.astype(np.int64).reshape(-1)
                 size = int(tokens.size)
                 if size == 0:
                     raise StepError(f"slot {slot} brings no token; leave idle sequences out of the step")
@@ -140,13 +142,24 @@ class Engine:
         ledger = self.cache.ledger
         for slot, length in checked["new_lengths"].items():
             ledger.reserve(slot, length)
-        plan = StepPlan(checked["slots"], checked["starts"], checked["counts"], checked["ids"],
-                        checked["wanted"], [self.cache.blocks(s) for s in checked["slots"]],
-                        self.cache.max_blocks)
-        if self.use_graphs:
-            logits = self._run_from_graph(plan, readout=bool(checked["wanted"]))
-        else:
-            logits = self._run_eager(plan, want_logits=bool(checked["wanted"]))
+        try:
+            plan = StepPlan(checked["slots"], checked["starts"], checked["counts"], checked["ids"],
+                            checked["wanted"], [self.cache.blocks(s) for s in checked["slots"]],
+                            self.cache.max_blocks)
+            if self.use_graphs:
+                logits = self._run_from_graph(plan, readout=bool(checked["wanted"]))
+            else:
+                logits = self._run_eager(plan, want_logits=bool(checked["wanted"]))
+        except BaseException:
+            # A pass that fails half-way (a kernel refuses its operands, a workspace cannot grow, the
+            # library reports an error) leaves every sequence as long as it was: the blocks reserved
+            # for this step go back, and what the pass wrote lies beyond the committed lengths, where
+            # nothing reads (src/models/llama/model/decode.rs:38-41; the reference's test of it is
+            # decode_tests.rs:762).  Fixed-size state is written by a mixer only after its own
+            # kernels were launched; a model that keeps such state is told to drop the sequences.
+            for slot in checked["new_lengths"]:
+                ledger.truncate(slot, ledger.lengths[slot])
+            raise
         for slot, length in checked["new_lengths"].items():
             ledger.commit(slot, length)
         self.steps_run += 1

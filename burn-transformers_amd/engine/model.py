@@ -41,7 +41,7 @@ class CausalLM:
         self.readout = build_part("readout", plan.readout, store)
         self.schedule = list(plan.schedule)
         self._check_schedule()
-        head_dims = sorted({d for block in self.blocks for d in block.parts["mixer"].head_dims()})
+        head_dims = sorted({d for block in self.blocks for mixer in block.mixers() for d in mixer.head_dims()})
         K.prepare(self.dtype, head_dims)
 
     def _check_schedule(self):
@@ -54,8 +54,7 @@ class CausalLM:
                                  f"the model has {len(self.blocks)}")
             if entry.cache is None:
                 continue
-            mixer = self.blocks[entry.layer].parts["mixer"]
-            specs = (mixer.kv_spec(), mixer.state_spec())
+            specs = self.blocks[entry.layer].cache_needs()
             if entry.writes:
                 if entry.cache in writers:
                     raise ValueError(f"cache entry {entry.cache} has two writers in the schedule")

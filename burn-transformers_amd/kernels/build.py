@@ -57,9 +57,24 @@ def _hash(name):
     return digest.hexdigest()
 
 
+def _own_private(path):
+    """True for a folder that belongs to this user and that nobody else can write to.  The
+    per-user fallback has a name anyone can guess and lies in a folder everyone can write to:
+    a library found there is loaded into this process, so a folder that somebody else made, or
+    can write to, is never read from and never written to."""
+    try:
+        status = os.stat(path, follow_symlinks=False)
+    except OSError:
+        return False
+    import stat
+    return stat.S_ISDIR(status.st_mode) and status.st_uid == os.getuid() and not (status.st_mode & 0o022)
+
+
 def _writable(path):
     try:
-        os.makedirs(path, exist_ok=True)
+        os.makedirs(path, mode=0o700, exist_ok=True)
+        if path == lib_dirs()[1] and not _own_private(path):
+            return False
         probe = os.path.join(path, f".probe-{os.getpid()}-{threading.get_ident()}")
         with open(probe, "w"):
             pass
@@ -76,7 +91,10 @@ def lib_dirs():
 
 
 def _find(name, wanted_hash):
-    for folder in lib_dirs():
+    package_dir, fallback = lib_dirs()
+    for folder in (package_dir, fallback):
+        if folder == fallback and not _own_private(folder):
+            continue
         lib = os.path.join(folder, name + ".so")
         stamp = os.path.join(folder, name + ".hash")
         try:

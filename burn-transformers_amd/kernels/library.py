@@ -214,7 +214,7 @@ def prepare(dtype, head_dims=()):
         if os.environ.get(PRODUCTS_ENV, "") != "own":
             names.append("gemm_library")
         names += [f"attention_bf16_hd{size}" for size in head_dims]
-    elif any(size <= 128 for size in head_dims):
+    elif any(size <= 128 and size % 16 == 0 for size in head_dims):
         names.append("attention_f32")
     with _lock:
         build.ensure_many(names)        # what is missing is compiled side by side
@@ -533,7 +533,7 @@ def attention(args, dtype, decode, impl="auto"):
         if code == BFLOAT16:
             impl = "mfma"
         else:
-            impl = "tiled" if args.kv.head_dim <= 128 and args.ldq % 4 == 0 else "plain"
+            impl = "tiled" if args.kv.head_dim <= 128 and args.kv.head_dim % 16 == 0 and args.ldq % 4 == 0 else "plain"
     if impl == "plain":
         lib = _module("core")
         _check(lib, lib.bt_attention_plain(_stream(), code, args))

@@ -15,6 +15,8 @@ Formulas: src/attention.rs:481-513 (projections), src/attention/dispatch.rs:314-
 output projection).
 """
 
+import torch
+
 from ..cache.storage import KVSpec
 from ..kernels import library as K
 from .base import Mixer, compute_units, packed_for_stream
@@ -41,8 +43,8 @@ class CausalSelfAttention(Mixer):
         self.head_dim, self.scale, self.window = p["head_dim"], float(p["scale"]), int(p.get("window") or 0)
         if not p.get("causal", True):
             raise ValueError("attention: only causal attention runs from a cache")
-        if self.head_dim % 16 != 0:
-            raise ValueError(f"attention: head size {self.head_dim} must be a multiple of 16")
+        if self.head_dim <= 0:
+            raise ValueError(f"attention: head size {self.head_dim} must be positive")
         if self.heads % self.kv_heads != 0:
             raise ValueError(f"attention: {self.heads} query heads cannot share {self.kv_heads} key/value heads")
         self.n_q, self.n_kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
@@ -55,6 +57,20 @@ class CausalSelfAttention(Mixer):
             raise ValueError(f"attention: output projection is {tuple(self.out_weight.shape)}, "
                              f"expected {(self.width, self.n_q)}")
 
+        # The MFMA kernels take head sizes in steps of 16 (bfloat16: up to 128).  In float32 every other
+        # size (any divisor of the width is a valid configuration, src/models/gpt2.rs:279-281) runs on
+        # the plain product and the plain attention kernel, which take any head size up to 256;
+        # bfloat16 has no such kernels and says so here, before anything is built.
+        bf16 = self.qkv_weight.dtype == torch.bfloat16
+        if bf16 and (self.head_dim % 16 != 0 or self.head_dim > 128):
+            raise ValueError(f"attention: the bfloat16 kernels take head sizes 16, 32, ... 128, not {self.head_dim}; "
+                             f"load the model with dtype float32, which takes any head size up to 256")
+        if self.head_dim > 256:
+            raise ValueError(f"attention: head size {self.head_dim} is beyond 256, the most any kernel here takes")
+        self.plain_only = self.head_dim % 16 != 0
+        if self.plain_only:
+            self.takes_deferred_norm = False       # the plain product reads row-major, normalised rows
+
         # second copies for decode steps, which read the weights and little else
         self.qkv_packed = K.PackedWeight(self.qkv_weight) if self.qkv_weight.is_cuda else None
         self.out_packed = packed_for_stream(self.out_weight) if self.out_weight.is_cuda else None
@@ -63,7 +79,7 @@ class CausalSelfAttention(Mixer):
         return KVSpec(self.kv_heads, self.head_dim, self.window)
 
     def head_dims(self):
-        return (self.head_dim,)
+        return () if self.plain_only else (self.head_dim,)
 
     def decode_runs(self, step, device):
         """Into how many runs a decode step's keys are cut: planned for the step's class of
@@ -92,7 +108,7 @@ class CausalSelfAttention(Mixer):
             q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
             K.gemm(h, self.qkv_weight,
                    K.epilogue_qkv(q, self.n_q, self.n_kv, kv, step.tok_seq, step.tok_pos, self.qkv_bias),
-                   packed=self.qkv_packed)
+                   packed=self.qkv_packed, impl="plain" if self.plain_only else "auto")
         else:   # the keys and values of another layer are read; only the queries are projected
             q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
             bias = self.qkv_bias[:self.n_q] if self.qkv_bias is not None else None
@@ -107,5 +123,5 @@ class CausalSelfAttention(Mixer):
             partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                 self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial)
-        K.attention(args, step.dtype, step.decode)
+        K.attention(args, step.dtype, step.decode, impl="plain" if self.plain_only else "auto")
         stream.add_product(step, mixed, self.out_weight, self.out_bias, packed=self.out_packed)

@@ -171,8 +171,30 @@ class Readout(Part):
 
 
 class Block:
+    """An arrangement of parts.  ``ROLES`` maps the block's own names for its parts to the registry
+    each is looked up in ("mixer", "feed_forward", "norm"); the names are the block's business, and
+    the engine asks the block, not the names, what it needs."""
+
+    ROLES = {}
+
     def __init__(self, parts):
         self.parts = parts
+
+    def mixers(self):
+        """The parts of this block that mix tokens (they say what the cache has to keep and which
+        kernels have to be built), whatever the block calls them."""
+        return [part for part in self.parts.values() if isinstance(part, Mixer)]
+
+    def cache_needs(self):
+        """(KVSpec or None, StateSpec or None): what one run of this block keeps in its cache entry.
+        A block has one cache entry per run, so at most one of its mixers may keep keys and values
+        and at most one fixed-size state."""
+        kv = [spec for spec in (mixer.kv_spec() for mixer in self.mixers()) if spec is not None]
+        state = [spec for spec in (mixer.state_spec() for mixer in self.mixers()) if spec is not None]
+        if len(kv) > 1 or len(state) > 1:
+            raise ValueError(f"{type(self).__name__}: a block's run has one cache entry, but several of its "
+                             f"mixers keep keys and values or state; give each of them a layer of its own")
+        return (kv[0] if kv else None, state[0] if state else None)
 
     def forward(self, stream, step, memory):
         raise NotImplementedError

@@ -14,8 +14,10 @@ TINY_A = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer":
           "n_inner": 256, "vocab_size": 1000, "n_positions": 128, "activation_function": "gelu_new",
           "layer_norm_epsilon": 1e-5, "scale_attn_by_inverse_layer_idx": False}
 TINY_B = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 3, "n_embd": 96, "n_head": 2,
-          "n_inner": 320, "vocab_size": 517, "n_positions": 192, "activation_function": "gelu",
+          "n_inner": 320, "vocab_size": 517, "n_positions": 64, "activation_function": "gelu",
           "layer_norm_epsilon": 1e-6, "scale_attn_by_inverse_layer_idx": True}
+# the same with room for sequences that cross several blocks of the cache
+TINY_BW = dict(TINY_B, n_positions=192)
 # an inner width that is odd, one head size, one layer: sizes the 16-byte loads of the kernels do not divide
 TINY_C = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 1, "n_embd": 32, "n_head": 2,
           "n_inner": 37, "vocab_size": 131, "n_positions": 80, "activation_function": "gelu_new",
@@ -24,7 +26,7 @@ TINY_C = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer":
 TINY_L = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "n_embd": 96, "n_head": 3,
           "n_inner": 128, "vocab_size": 211, "n_positions": 4300, "activation_function": "gelu_new",
           "layer_norm_epsilon": 1e-5, "scale_attn_by_inverse_layer_idx": False}
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "L": (TINY_L, 3)}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "BW": (TINY_BW, 1), "C": (TINY_C, 2), "L": (TINY_L, 3)}
 
 _folders = {}
 
@@ -61,6 +63,8 @@ def prompts_for(name, lengths, seed=0):
 
 def tolerance(dtype, reference):
     """Largest allowed absolute error of logits: float32 differs from float64 by summation order
-    only; bfloat16 rounds every activation to 8 bits of mantissa."""
+    only; bfloat16 rounds every activation between two kernels to 8 bits of mantissa (relative
+    2^-9 = 2e-3 each), which through the few layers of these models measures 2e-3 to 4e-3 of the
+    largest logit; the bound is twice that."""
     scale = float(reference.abs().max())
-    return 2e-5 + 1e-5 * scale if dtype == "float32" else 2.5e-2 * scale
+    return 2e-5 + 1e-5 * scale if dtype == "float32" else 8e-3 * scale

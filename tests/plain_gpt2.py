@@ -1,7 +1,7 @@
 """Plain, slow GPT-2 used only as the oracle of the tests.
 
 Whole sequences, no cache, one sequence at a time, one function per part, written from
-the formulas of the reference (cited as path:line below /root/reference) and sharing no
+the formulas of the reference (cited as path:line of the reference) and sharing no
 code with the product path.  Weights are a dict of torch tensors under the checkpoint's
 own names and Conv1D ``[in, out]`` layout (``h.N.attn.c_attn.weight`` ...).  Everything
 is evaluated in ``dtype`` (float64 unless asked otherwise).
@@ -131,11 +131,22 @@ def block(x, w, layer, cfg, taps=None):
     return y + f
 
 
+class _Converted:
+    """The weights in ``dtype``, each tensor converted when it is used (a model of a billion
+    parameters is not held a second time)."""
+
+    def __init__(self, tensors, dtype):
+        self.tensors, self.dtype = tensors, dtype
+
+    def __getitem__(self, name):
+        return self.tensors[name].to(self.dtype)
+
+
 def forward(ids, w, cfg, dtype=torch.float64, taps=None, rows=None):
     """Logits [S, V] of one whole sequence: embed, blocks, ln_f, tied readout
     (src/models/gpt2/model.rs:385-420, 500-513).  With ``rows``, only those positions are read out:
     the selection comes after the final norm and before the product (src/models/shared/logits.rs:58-80)."""
-    w = {name: t.to(dtype) for name, t in w.items()}
+    w = _Converted(w, dtype)
     ids = torch.as_tensor(ids, dtype=torch.long)
     x = embed(ids, torch.arange(ids.numel()), w["wte.weight"], w["wpe.weight"])
     if taps is not None:

@@ -42,6 +42,7 @@ def test_aliases_unknown_keys_and_wrappers():
     ({"reorder_and_upcast_attn": True}, "reorder_and_upcast_attn"),
     ({"add_cross_attention": True}, "add_cross_attention"),
     ({"tie_word_embeddings": False}, "tie_word_embeddings"),
+    ({"causal": False}, "causal"),
     ({"n_inner": 0}, "n_inner"),
     ({"activation_function": "relu"}, "activation_function"),
     ({"n_embd": "wide"}, "n_embd"),

@@ -463,7 +463,7 @@ def test_attention_mfma(q_heads, kv_heads, hd, totals, counts, window):
 def test_attention_finds_one_far_key_among_hundreds():
     """One key far back is made to dominate; an off-by-one in block or tile addressing loses it."""
     hd, total = 64, 700
-    for dt, target in [(torch.bfloat16, t) for t in (0, 63, 64, 333, 698)] + [(torch.float32, t) for t in (0, 64, 333, 698)]:
+    for dt, target in [(torch.bfloat16, t) for t in (0, 63, 64, 333, 671, 672, 698, 699)] + [(torch.float32, t) for t in (0, 64, 333, 698, 699)]:
         case = PagedCase([total], [1], 1, hd, dt, DEV, seed=target)
         q = torch.zeros(1, hd)
         q[0, 3] = 8.0
@@ -482,6 +482,79 @@ def test_attention_finds_one_far_key_among_hundreds():
                                     1, 1, 1, 1.0, 0)
             K.attention(args, dt, decode=decode, impl=impl)
             assert rel_err(out, want) < 1e-2, (target, impl, decode)
+
+
+def _dominant_target(row, pos):
+    """The one key query ``row`` at position ``pos`` looks at: its own position, the one before, the
+    first key of its block of 64, the last key of the tile of 32 before its own, key 0, or a key
+    of an odd block of 64 far back."""
+    kind = row % 6
+    if kind == 0:
+        return pos
+    if kind == 1:
+        return max(pos - 1, 0)
+    if kind == 2:
+        return pos // 64 * 64
+    if kind == 3:
+        return max(pos // 32 * 32 - 1, 0)
+    if kind == 4:
+        return 0
+    return 64 * (2 * (pos // 128) - 1) + pos % 64 if pos >= 128 else pos // 2
+
+
+@pytest.mark.parametrize("dtype,q_heads,kv_heads,hd,totals,counts", [
+    ("bfloat16", 2, 2, 64, [700, 450, 333], [517, 450, 70]),        # chunks that start at 183 and 263
+    ("bfloat16", 4, 2, 32, [700, 450, 333], [517, 450, 70]),
+    ("bfloat16", 4, 4, 64, [600] * 13 + [100], [600] * 13 + [100]),   # more query tiles than compute units
+    ("bfloat16", 2, 1, 128, [300, 129], [171, 129]),
+    ("float32", 2, 2, 64, [700, 450, 333], [517, 450, 70]),
+    ("float32", 3, 3, 48, [300, 129], [171, 129]),
+])
+def test_prefill_attention_every_query_finds_its_one_key(dtype, q_heads, kv_heads, hd, totals, counts):
+    """Every query of a prompt (or chunk) is given ONE key that takes all the weight, at a place
+    chosen to sit on the edges of the kernels' tiles: on the diagonal, just before it, at the first
+    key of the query's block, at the last key of the tile before, at key 0, in an odd block far
+    back.  A key that a tile edge, the bound of the unmasked tiles, or the hand-over between the two
+    halves of a work-group loses or counts twice changes the query's output from that key's value
+    row to some other's, which no tolerance hides."""
+    dt = DTYPES[dtype]
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=31, poison=True)
+    group = q_heads // kv_heads
+    q = torch.zeros(case.n_tokens, q_heads * hd)
+    row = 0
+    for s, (total, count) in enumerate(zip(totals, counts)):
+        keys = case.k_rows[s].float().view(total, kv_heads, hd)
+        keys = keys / keys.norm(dim=-1, keepdim=True)          # unit keys: a key's score with itself is the largest
+        case.k_rows[s] = keys.reshape(total, kv_heads * hd).to(dt)
+        stored = case.k_rows[s].float().view(total, kv_heads, hd)
+        for i in range(count):
+            pos = total - count + i
+            for head in range(q_heads):
+                q[row, head * hd:(head + 1) * hd] = stored[_dominant_target(row + head, pos), head // group]
+            row += 1
+    seq = torch.cat([torch.full((t,), s, dtype=torch.int32) for s, t in enumerate(totals)]).to(DEV)
+    pos = torch.cat([torch.arange(t, dtype=torch.int32) for t in totals]).to(DEV)
+    K.kv_copy(torch.cat(case.k_rows).to(DEV), torch.cat(case.v_rows).to(DEV), seq, pos, case.view(), True)
+    q = q.to(dt).to(DEV)
+    scale = 60.0           # the target scores 60, any other key 60 cos(angle): below 40 among random directions
+    want = case.reference(q, q_heads, scale)
+    # the premise: every output row IS (nearly) one value row
+    row = 0
+    for s, (total, count) in enumerate(zip(totals, counts)):
+        values = case.v_rows[s].double().view(total, kv_heads, hd)
+        for i in range(0, count, 37):
+            target = _dominant_target(row + i, total - count + i)
+            assert (want[row + i, :hd] - values[target, 0]).abs().max() < 2e-2
+        row += count
+    impl = "mfma" if dtype == "bfloat16" else "tiled"
+    out = torch.full((case.n_tokens, q_heads * hd), float("nan"), dtype=dt, device=DEV)
+    args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                            q_heads, len(totals), max(counts), scale, 0)
+    K.attention(args, dt, decode=False, impl=impl)
+    error = (out.detach().cpu().double() - want).abs().max(dim=1).values
+    worst = int(error.argmax())
+    assert float(error.max()) < (2e-2 if dtype == "bfloat16" else 1e-4), \
+        f"query row {worst} (position {int(case.tok_pos[worst])} of sequence {int(case.tok_seq[worst])}) is off by {float(error.max())}"
 
 
 @pytest.mark.parametrize("dtype,hd,window", [("bfloat16", 64, 0), ("bfloat16", 32, 0), ("bfloat16", 64, 3000),

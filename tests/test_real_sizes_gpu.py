@@ -97,6 +97,29 @@ def test_whole_request(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_prompts_in_chunks_that_start_off_the_block_grid(dtype):
+    """Two requests fed in chunks of 200 and 130 tokens: chunks start at 200, 400, 600 and at 130,
+    260, ..., none a multiple of the cache's blocks of 64 or the kernels' tiles of 128 queries."""
+    engine = engine_for(dtype)
+    requests = [request(700, seed=2), request(520, seed=5)]
+    chunks, fed, slots = [200, 130], [0, 0], [engine.open(), engine.open()]
+    got, rows = [[], []], [[], []]
+    while any(f < len(r) for f, r in zip(fed, requests)):
+        live = [i for i in range(2) if fed[i] < len(requests[i])]
+        entries = [(slots[i], requests[i][fed[i]:fed[i] + chunks[i]]) for i in live]
+        wants = [[0, len(e[1]) // 2, len(e[1]) - 1] for e in entries]
+        logits = engine.step(entries, want=wants).clone()
+        for n, i in enumerate(live):
+            got[i].append(logits[3 * n:3 * n + 3])
+            rows[i] += [fed[i] + w for w in wants[n]]
+            fed[i] += len(entries[n][1])
+    for i, r in enumerate(requests):
+        check(torch.cat(got[i]), plain_rows(r, rows[i]), dtype, f"request {i} in chunks of {chunks[i]}")
+    for slot in slots:
+        engine.close(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_last_32_tokens_one_by_one_up_to_the_position_limit(dtype):
     engine = engine_for(dtype)
     ids = request(1024, seed=3)

@@ -160,10 +160,10 @@ def test_generation_with_penalties_follows_the_plain_loop():
 
 
 def test_sampled_generation_with_truncation_is_reproducible_and_respects_top_k():
-    folder, cfg, _ = model_folder("B")
+    folder, cfg, _ = model_folder("BW")
     model = bt.load_model(folder, dtype="bfloat16")
     engine = bt.Engine(model, max_tokens=1024)
-    prompts = prompts_for("B", [5, 40], seed=2)
+    prompts = prompts_for("BW", [5, 40], seed=2)
     config = bt.GenerationConfig(max_new_tokens=12, strategy="sample", temperature=0.9, top_k=1, top_p=0.9, seed=4)
     sampled = bt.generate(engine, prompts, config)
     greedy = bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=12))

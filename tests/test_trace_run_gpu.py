@@ -86,7 +86,7 @@ def compare(name, dtype, got, want, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,lengths", [("A", [40, 128, 65]), ("B", [33, 192, 100])])
+@pytest.mark.parametrize("name,lengths", [("A", [40, 128, 65]), ("BW", [33, 192, 100])])
 def test_replay_whole_tail_and_batches(name, dtype, lengths, tmp_path):
     requests = prompts_for(name, lengths, seed=50)
     reference = [plain_logits(name, r) for r in requests]

@@ -63,9 +63,9 @@ def request(length, seed):
 
 def oracle(ids):
     """float64 logits of every position of the request (kept: both precisions ask for the same)."""
+    xl_weights()
     key = tuple(ids)
     if key not in _xl["oracle"]:
-        xl_weights()
         print(f"[depth] plain forward of {len(ids)} tokens through 48 layers", flush=True)
         _xl["oracle"][key] = plain.forward(ids, _xl["wide"], XL)
     return _xl["oracle"][key]

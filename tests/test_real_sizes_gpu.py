@@ -63,11 +63,21 @@ def plain_rows(ids, rows):
     return plain.forward(ids, weights, WIDE, rows=rows)
 
 
+# bfloat16 under sharpened attention: a score of magnitude 15 computed from queries and keys rounded
+# to 8 bits is off by about 15 * 2^-8 = 0.06, so a weight of the softmax by 6 %, where the
+# initialiser's nearly uniform attention would hide both this and a lost key.  Measured over this
+# file's cases: 1.2e-2 to 1.6e-2 of the largest logit.  What a tolerance of this size could hide
+# is covered by the tests of the attention kernels in which one key takes all the weight.
+BF16_BOUND = 2.5e-2
+
+
 def check(got, want, dtype, what):
     got = got.detach().cpu().double()
     err = float((got - want).abs().max())
     assert torch.isfinite(got).all(), what
-    assert err <= tolerance(dtype, want), f"{what}: max abs error {err} > {tolerance(dtype, want)}"
+    bound = tolerance(dtype, want) if dtype == "float32" else BF16_BOUND * float(want.abs().max())
+    print(f"[real sizes] {what} ({dtype}): max abs error {err:.3g}, {err / float(want.abs().max()):.3g} of the largest logit", flush=True)
+    assert err <= bound, f"{what}: max abs error {err} > {bound}"
 
 
 def test_attention_of_the_wide_model_is_peaked():

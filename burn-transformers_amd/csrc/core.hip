@@ -10,9 +10,12 @@
 
 #include <float.h>
 
+#include <mutex>
+
 #include "host.h"
 #include "epilogue.h"
 #include "attention.h"
+#include "no_alloc.h"
 
 // ---------------------------------------------------------------------------------------------
 // Embedding: x[t] = table[ids[t]] (+ positions[pos[t]]), written as 32-bit residual stream.
@@ -783,6 +786,10 @@ BT_EXPORT int64_t bt_sample_workspace_bytes(int rows, int vocab) {
   return (int64_t)rows * sample_chunks(vocab > 0 ? vocab : 1) * sizeof(SamplePartial);
 }
 
+static int launch_sample(void* stream, const float* logits, int64_t ld, int rows, int vocab, int sample,
+                         float temperature, uint64_t seed, uint64_t first_draw, const int* draw_rows,
+                         int* ids, float* logp, void* workspace);
+
 BT_EXPORT int bt_sample(void* stream, const float* logits, int64_t ld, int rows, int vocab, int sample,
                         float temperature, uint64_t seed, uint64_t first_draw, const int* draw_rows,
                         int* ids, float* logp, void* workspace) {
@@ -790,6 +797,64 @@ BT_EXPORT int bt_sample(void* stream, const float* logits, int64_t ld, int rows,
   if (vocab <= 0) BT_REFUSE("sample: vocabulary %d must be positive", vocab);
   if (sample && !(temperature > 0.f)) BT_REFUSE("sample: temperature %g must be positive", (double)temperature);
   if (workspace == nullptr) BT_REFUSE("sample: no workspace");
+  return launch_sample(stream, logits, ld, rows, vocab, sample, temperature, seed, first_draw, draw_rows, ids, logp,
+                       workspace);
+}
+
+// The same without a workspace argument, for callers that cannot allocate (no_alloc.h): the
+// partial results live in an array of the library's own on each GPU.  In host code the array's
+// name is only a stand-in for the symbol; its address in a device's memory is looked up once per
+// device, with that device current, and every use below goes through that address.
+static __device__ __align__(256) unsigned char scratch[BT_NO_ALLOC_SCRATCH_BYTES];
+
+#define BT_NO_ALLOC_MAX_DEVICES 64
+static void* scratch_address[BT_NO_ALLOC_MAX_DEVICES];     // by device number; null = not looked up yet
+static std::mutex scratch_lock;
+
+static int scratch_on_current_device(void** address) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) BT_REFUSE("sample_no_alloc: no current device: %s", hipGetErrorString(err));
+  if (device < 0 || device >= BT_NO_ALLOC_MAX_DEVICES)
+    BT_REFUSE("sample_no_alloc: device %d is beyond the %d this library keeps an address for", device, BT_NO_ALLOC_MAX_DEVICES);
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_address[device] == nullptr) {
+    void* found = nullptr;
+    err = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || found == nullptr) {
+      bt_set_error("sample_no_alloc: the scratch array has no address on device %d: %s", device, hipGetErrorString(err));
+      return BT_HIP_ERROR;
+    }
+    scratch_address[device] = found;
+  }
+  *address = scratch_address[device];
+  return BT_OK;
+}
+
+BT_EXPORT int64_t bt_sample_no_alloc_capacity(void) { return BT_NO_ALLOC_SCRATCH_BYTES / (int64_t)sizeof(SamplePartial); }
+
+BT_EXPORT int bt_sample_no_alloc(void* stream, const float* logits, int64_t ld, int rows, int vocab, int sample,
+                                 float temperature, uint64_t seed, uint64_t first_draw, const int* draw_rows,
+                                 int* ids, float* logp) {
+  if (rows <= 0) return BT_OK;
+  if (vocab <= 0) BT_REFUSE("sample_no_alloc: vocabulary %d must be positive", vocab);
+  if (sample && !(temperature > 0.f)) BT_REFUSE("sample_no_alloc: temperature %g must be positive", (double)temperature);
+  if (logits == nullptr || ids == nullptr || logp == nullptr) BT_REFUSE("sample_no_alloc: missing operand");
+  const int64_t records = (int64_t)rows * sample_chunks(vocab);
+  if (records > bt_sample_no_alloc_capacity())
+    BT_REFUSE("sample_no_alloc: %d rows of %d logits need %lld partial results, the fixed scratch array holds %lld "
+              "(use bt_sample with a workspace of bt_sample_workspace_bytes)",
+              rows, vocab, (long long)records, (long long)bt_sample_no_alloc_capacity());
+  void* partials = nullptr;
+  int rc = scratch_on_current_device(&partials);
+  if (rc) return rc;
+  return launch_sample(stream, logits, ld, rows, vocab, sample, temperature, seed, first_draw, draw_rows, ids, logp,
+                       partials);
+}
+
+static int launch_sample(void* stream, const float* logits, int64_t ld, int rows, int vocab, int sample,
+                         float temperature, uint64_t seed, uint64_t first_draw, const int* draw_rows,
+                         int* ids, float* logp, void* workspace) {
   const int chunks = sample_chunks(vocab);
   const int chunk_len = (vocab + chunks - 1) / chunks;
   // the logits are divided by the temperature only when sampling

@@ -19,7 +19,7 @@ import time
 PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
-HEADERS = ("common.h", "host.h", "epilogue.h", "attention.h")
+HEADERS = ("common.h", "host.h", "epilogue.h", "attention.h", "no_alloc.h")
 # -packed-fp32-ops is switched off for every kernel: some packed 32-bit forms have produced
 # wrong values on this hardware generation.
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=" + ARCH, "-fPIC", "-shared",

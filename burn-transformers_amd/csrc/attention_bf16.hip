@@ -28,6 +28,7 @@
 
 #include "host.h"
 #include "attention.h"
+#include "calls.h"
 
 #ifndef BT_HEAD_DIM
 #error "compile with -DBT_HEAD_DIM=<multiple of 16>"
@@ -816,3 +817,7 @@ BT_EXPORT int bt_attention_decode_bf16(void* stream, const AttnArgs* args) {
   }
   return bt_check_launch("attention_decode_bf16");
 }
+
+// The same entry points with their arguments as one structure (calls.h), for launch lists.
+BT_EXPORT int bt_attention_prefill_bf16_call(void* stream, const AttentionCall* c) { return bt_attention_prefill_bf16(stream, &c->args); }
+BT_EXPORT int bt_attention_decode_bf16_call(void* stream, const AttentionCall* c) { return bt_attention_decode_bf16(stream, &c->args); }

@@ -26,6 +26,7 @@
 
 #include "host.h"
 #include "attention.h"
+#include "calls.h"
 
 #define F32_QUERIES 32
 #define F32_WAVE_QUERIES 8
@@ -398,3 +399,6 @@ BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
   }
   return bt_check_launch("attention_f32");
 }
+
+// The same entry points with their arguments as one structure (calls.h), for launch lists.
+BT_EXPORT int bt_attention_f32_call(void* stream, const AttentionCall* c) { return bt_attention_f32(stream, &c->args); }

@@ -15,6 +15,7 @@
 #include "host.h"
 #include "epilogue.h"
 #include "attention.h"
+#include "calls.h"
 #include "no_alloc.h"
 
 // ---------------------------------------------------------------------------------------------
@@ -1199,4 +1200,26 @@ BT_EXPORT int bt_count_tokens(void* stream, int* counts, int64_t ld, const int* 
   if (n <= 0) return BT_OK;
   hipLaunchKernelGGL(count_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, counts, ld, rows, ids, n);
   return bt_check_launch("count_tokens");
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same entry points with their arguments as one structure (calls.h), for launch lists.
+// ---------------------------------------------------------------------------------------------
+BT_EXPORT int bt_embed_call(void* stream, const EmbedCall* c) {
+  return bt_embed(stream, c->dtype, c->ids, c->pos, c->table, c->positions, c->out, c->tokens, c->width);
+}
+BT_EXPORT int bt_add_norm_call(void* stream, const AddNormCall* c) {
+  return bt_add_norm(stream, c->out_dtype, c->x, c->delta, c->n_delta, c->delta_stride, c->bias, c->gamma, c->beta, c->eps,
+                     c->kind, c->out, c->rows, c->n_rows, c->width, c->write_back, c->out_rows);
+}
+BT_EXPORT int bt_gemm_plain_call(void* stream, const GemmCall* c) {
+  if (c->splits != 1 || c->has_norm || c->a_rows || c->packed_columns)
+    BT_REFUSE("gemm_plain: no split of K, no rows to normalise, no chunk-major rows and no packed weights");
+  return bt_gemm_plain(stream, c->dtype, c->A, c->lda, c->W, c->M, c->N, c->K, &c->epi);
+}
+BT_EXPORT int bt_attention_plain_call(void* stream, const AttentionCall* c) {
+  return bt_attention_plain(stream, c->dtype, &c->args);
+}
+BT_EXPORT int bt_kv_copy_call(void* stream, const KvCopyCall* c) {
+  return bt_kv_copy(stream, c->dtype, c->k_rows, c->v_rows, c->ld, c->tok_seq, c->tok_pos, &c->kv, c->tokens, c->to_cache);
 }

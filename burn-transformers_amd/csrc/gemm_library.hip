@@ -24,6 +24,7 @@
 
 #include "epilogue.h"
 #include "host.h"
+#include "calls.h"
 
 namespace {
 
@@ -203,4 +204,25 @@ BT_EXPORT int bt_gemm_library_bf16(void* stream, const void* A, int64_t lda, con
     if (rc) return rc;
   }
   return BT_OK;
+}
+
+// Whether the library has an algorithm for this product, found (and kept) without running anything:
+// what a launch list asks before it names the library for a product.
+BT_EXPORT int bt_gemm_library_plan(int64_t lda, int M, int N, int K, const Epilogue* epi) {
+  if (M <= 0) return BT_OK;
+  if (handle == nullptr) BT_REFUSE("gemm_library: the library has not been opened");
+  if (N <= 0 || K <= 0 || lda < K || epi->ldo < N) BT_REFUSE("gemm_library: sizes M %d N %d K %d do not fit the pitches", M, N, K);
+  if (epi->mode != EPI_STORE && epi->mode != EPI_RESIDUAL && epi->mode != EPI_F32 &&
+      !(epi->mode == EPI_ACT && epi->act == ACT_GELU_TANH))
+    BT_REFUSE("gemm_library: epilogue %d (activation %d) is not one the library has", epi->mode, epi->act);
+  if (plan_for(M < ROWS_PER_CALL ? M : ROWS_PER_CALL, N, K, lda, epi) == nullptr) return BT_REFUSED;
+  if (M > ROWS_PER_CALL && M % ROWS_PER_CALL != 0 && plan_for(M % ROWS_PER_CALL, N, K, lda, epi) == nullptr) return BT_REFUSED;
+  return BT_OK;
+}
+
+// The product with its arguments as one structure (calls.h), for launch lists.
+BT_EXPORT int bt_gemm_library_call(void* stream, const GemmCall* c) {
+  if (c->dtype != 1 || c->splits != 1 || c->has_norm || c->a_rows || c->packed_columns || c->epi.out_rows)
+    BT_REFUSE("gemm_library: bfloat16 row-major operands only, no split of K");
+  return bt_gemm_library_bf16(stream, c->A, c->lda, c->W, c->M, c->N, c->K, &c->epi);
 }

@@ -24,6 +24,7 @@
 
 #include "host.h"
 #include "epilogue.h"
+#include "calls.h"
 
 #define TILE_K 64            // bfloat16 values in a 128-byte row of an LDS tile
 #define TILE_ROW_BYTES 128
@@ -484,15 +485,6 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
 // statistics as wave reductions) and leaves them in LDS as bfloat16, where the multiplication
 // reads its operand.  The rows' loads are issued before the first batch of weights, so the
 // statistics are computed while the weights are on their way.
-struct NormOperand {
-  const float* x;        // [M][ldx] float32 rows
-  int64_t ldx;
-  const float* gamma;    // [K]
-  const float* beta;     // [K] or null
-  float eps;
-  int kind;              // 0: layer norm, 1: RMS norm
-};
-
 __device__ float bt_norm_zeros[4] = {0.f, 0.f, 0.f, 0.f};
 
 template <typename T, int MT, int NT, int U, int WAVES, int QPL = 0, bool CHUNKED = false>
@@ -898,4 +890,15 @@ BT_EXPORT int bt_gemm_skinny(void* stream, int dtype, const void* A, int64_t lda
     launch_skinny<bf16_t>((hipStream_t)stream, (const bf16_t*)A, lda, (const bf16_t*)W, M, N, K, *epi, splits, columns, packed, a_rows);
   }
   return bt_check_launch("gemm_skinny");
+}
+
+// The same entry points with their arguments as one structure (calls.h), for launch lists.
+BT_EXPORT int bt_gemm_tile_call(void* stream, const GemmCall* c) {
+  if (c->has_norm || c->a_rows || c->packed_columns)
+    BT_REFUSE("gemm_tile: no rows to normalise, no chunk-major rows and no packed weights");
+  return bt_gemm_tile(stream, c->dtype, c->A, c->lda, c->W, c->M, c->N, c->K, &c->epi, c->splits, c->variant);
+}
+BT_EXPORT int bt_gemm_skinny_call(void* stream, const GemmCall* c) {
+  return bt_gemm_skinny(stream, c->dtype, c->A, c->lda, c->W, c->M, c->N, c->K, &c->epi, c->splits, c->variant,
+                        c->has_norm ? &c->norm : nullptr, c->packed_columns, c->a_rows);
 }

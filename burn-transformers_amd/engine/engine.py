@@ -27,10 +27,13 @@ import numpy as np
 import torch
 
 from ..cache.storage import Cache
+from ..kernels import library as K
 from .step import BufferPool, Step, StepLayout, StepPlan
 
 _PINNED_RING = 4
 _MAX_GRAPHS = 48           # graphs kept; the one that was used longest ago goes first
+_MAX_PROGRAMS = 1024       # launch lists kept (a few hundred small structures each)
+_META_WORDS = 1 << 16      # first size of the device buffer of a step's integer tables
 
 
 class StepError(ValueError):
@@ -38,7 +41,7 @@ class StepError(ValueError):
 
 
 class Engine:
-    def __init__(self, model, max_tokens, max_slots=None, graphs=True):
+    def __init__(self, model, max_tokens, max_slots=None, graphs=True, programs=True):
         self.model = model
         self.device, self.dtype = model.device, model.dtype
         self.cache = Cache(model.kv_specs, model.state_specs, max_tokens, model.max_positions,
@@ -46,6 +49,12 @@ class Engine:
         self.pool = BufferPool(self.device)
         # a mixer that plans work on the host per step cannot be replayed from a graph
         self.use_graphs = graphs and all(mixer.graph_safe for block in model.blocks for mixer in block.mixers())
+        # Steps that are not replayed from a graph are kept as launch lists, one per shape, and walked
+        # in C++ (kernels.library.Program), if every part of the model only launches kernels
+        self.use_programs = programs and getattr(model, "recordable", False)
+        self._programs = {}                # shape -> (Program, logits), in order of last use
+        self._programs_generation = -1     # the workspace generation the lists were recorded for
+        self.program_runs = 0
         self._meta = None                  # device int32 buffer of eager steps
         self._pinned = []                  # ring of (pinned int32 tensor, event)
         self._pinned_next = 0
@@ -182,13 +191,51 @@ class Engine:
 
     def _run_eager(self, plan, want_logits=True):
         if self._meta is None or self._meta.numel() < plan.layout.total:
-            self._meta = torch.empty(max(plan.layout.total * 2, 4096), dtype=torch.int32, device=self.device)
+            self._meta = torch.empty(max(plan.layout.total * 2, _META_WORDS), dtype=torch.int32, device=self.device)
+            self._programs.clear()                        # they name the old tables
         self._upload(plan.host, self._meta)
+        if self.use_programs:
+            return self._run_program(plan, want_logits)
         step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
         if not want_logits:       # a step whose logits nobody wants still has to fill the cache
             self.model.forward(step, self.cache, readout=False)
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return self.model.forward(step, self.cache)
+
+    def _run_program(self, plan, readout):
+        """The step from its launch list: recorded the first time a shape comes (the parts run as
+        always, but every kernel call is kept instead of launched), walked in C++ every time.  A
+        list names workspaces by address, so a workspace that had to grow makes all lists stale."""
+        if self._programs_generation != self.pool.generation:
+            self._programs.clear()
+            self._programs_generation = self.pool.generation
+        key = (plan.layout.key(), plan.max_count, readout, plan.context_limit if plan.decode else 0)
+        held = self._programs.pop(key, None)
+        if held is None:
+            step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
+            for _ in range(4):
+                # a workspace that grows WHILE the list is recorded leaves its old address in the calls
+                # recorded before: record again, now that it is large enough from the start
+                generation = self.pool.generation
+                program = K.Program()
+                with program.recording():
+                    logits = self.model.forward(step, self.cache, readout=readout)
+                if self.pool.generation == generation:
+                    break
+            else:
+                raise RuntimeError("the workspaces of a step did not settle while its launch list was recorded")
+            if not readout:
+                logits = torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+            if self._programs_generation != self.pool.generation:      # recording made a workspace grow:
+                self._programs.clear()                                 # the lists before this one are stale
+                self._programs_generation = self.pool.generation
+            held = (program, logits)
+            while len(self._programs) >= _MAX_PROGRAMS:
+                self._programs.pop(next(iter(self._programs)))
+        self._programs[key] = held                        # (again) the most recently used
+        held[0].run()
+        self.program_runs += 1
+        return held[1]
 
     def _run_from_graph(self, plan, readout):
         # (parts plan decode steps by the class of context; steps with prompt tokens look the same in every class)

@@ -41,6 +41,9 @@ class CausalLM:
         self.readout = build_part("readout", plan.readout, store)
         self.schedule = list(plan.schedule)
         self._check_schedule()
+        # a step of this model can be kept as a launch list if every part only launches kernels
+        self.recordable = all(block.recordable() for block in self.blocks) and \
+            all(part.only_launches_kernels for part in (self.embedding, self.final_norm, self.readout))
         head_dims = sorted({d for block in self.blocks for mixer in block.mixers() for d in mixer.head_dims()})
         K.prepare(self.dtype, head_dims)
 

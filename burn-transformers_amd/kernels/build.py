@@ -19,7 +19,7 @@ import time
 PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
-HEADERS = ("common.h", "host.h", "epilogue.h", "attention.h", "no_alloc.h")
+HEADERS = ("common.h", "host.h", "epilogue.h", "attention.h", "calls.h", "no_alloc.h")
 # -packed-fp32-ops is switched off for every kernel: some packed 32-bit forms have produced
 # wrong values on this hardware generation.
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=" + ARCH, "-fPIC", "-shared",
@@ -40,11 +40,13 @@ def module_source(name):
         return name + ".hip", []
     if name == "gemm_library":      # host code around hipBLASLt, which it opens at run time
         return name + ".hip", ["-ldl"]
+    if name == "program":           # the host loop that walks a launch list: C++ only, no kernels
+        return name + ".cpp", []
     raise ValueError(f"unknown kernel module {name!r}")
 
 
 def all_modules():
-    return ["core", "gemm_mfma", "gemm_library", "attention_f32"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
+    return ["core", "gemm_mfma", "gemm_library", "program", "attention_f32"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
 
 
 def _hash(name):

@@ -56,6 +56,37 @@ class NormOperand(ctypes.Structure):
                 ("kind", _c_int)]
 
 
+class EmbedCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("width", _c_int), ("ids", _c_ptr), ("pos", _c_ptr),
+                ("table", _c_ptr), ("positions", _c_ptr), ("out", _c_ptr)]
+
+
+class AddNormCall(ctypes.Structure):
+    _fields_ = [("out_dtype", _c_int), ("n_delta", _c_int), ("kind", _c_int), ("n_rows", _c_int), ("width", _c_int),
+                ("write_back", _c_int), ("out_rows", _c_int), ("eps", _c_float), ("x", _c_ptr), ("delta", _c_ptr),
+                ("delta_stride", _c_i64), ("bias", _c_ptr), ("gamma", _c_ptr), ("beta", _c_ptr), ("out", _c_ptr),
+                ("rows", _c_ptr)]
+
+
+class GemmCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("M", _c_int), ("N", _c_int), ("K", _c_int), ("splits", _c_int), ("variant", _c_int),
+                ("packed_columns", _c_int), ("a_rows", _c_int), ("has_norm", _c_int), ("A", _c_ptr), ("lda", _c_i64),
+                ("W", _c_ptr), ("epi", Epilogue), ("norm", NormOperand)]
+
+
+class AttentionCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("args", AttnArgs)]
+
+
+class KvCopyCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("to_cache", _c_int), ("k_rows", _c_ptr), ("v_rows", _c_ptr),
+                ("ld", _c_i64), ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView)]
+
+
+class LaunchEntry(ctypes.Structure):
+    _fields_ = [("call", _c_ptr), ("args", _c_ptr)]
+
+
 class Chunked:
     """Activations of a step of few rows kept chunk-major: the chunks of 64 bytes of the columns (32
     bfloat16 or 16 float32 values) one after the other, each with that chunk of every row,
@@ -119,25 +150,11 @@ class Normalized:
         return rows <= cls.MAX_ROWS and width <= cls.MAX_WIDTH and width % 8 == 0
 
 
-# Argument types of the entry points a step calls hundreds of times: with them declared, plain
-# Python integers, None and structures can be passed as they are, and a wrong count of arguments
-# is an error at the call instead of garbage in a register.
-_P = ctypes.POINTER
-_SIGNATURES = {
-    "bt_embed": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int],
-    "bt_add_norm": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_int,
-                    _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int],
-    "bt_gemm_plain": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue)],
-    "bt_gemm_tile": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue), _c_int, _c_int],
-    "bt_gemm_skinny": [_c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue), _c_int, _c_int,
-                       _P(NormOperand), _c_int, _c_int],
-    "bt_gemm_library_bf16": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _P(Epilogue)],
-    "bt_attention_plain": [_c_ptr, _c_int, _P(AttnArgs)],
-    "bt_attention_f32": [_c_ptr, _P(AttnArgs)],
-    "bt_attention_prefill_bf16": [_c_ptr, _P(AttnArgs)],
-    "bt_attention_decode_bf16": [_c_ptr, _P(AttnArgs)],
-    "bt_kv_copy": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _P(KvView), _c_int, _c_int],
-}
+# Every kernel of a step is called through its structure form, bt_<kernel>_call(stream, structure)
+# (csrc/calls.h): the same pair can be called now or kept in a launch list (:class:`Program`).
+_CALLS = ("bt_embed_call", "bt_add_norm_call", "bt_gemm_plain_call", "bt_gemm_tile_call", "bt_gemm_skinny_call",
+          "bt_gemm_library_call", "bt_attention_plain_call", "bt_attention_f32_call",
+          "bt_attention_prefill_bf16_call", "bt_attention_decode_bf16_call", "bt_kv_copy_call")
 
 _modules = {}
 _lock = threading.Lock()
@@ -155,10 +172,11 @@ def _module(name):
                 lib = ctypes.CDLL(path)
             except OSError as error:
                 raise RuntimeError(f"cannot load the kernel library {path}: {error}") from error
-            lib.bt_last_error.restype = ctypes.c_char_p
-            for entry, types in _SIGNATURES.items():
+            if name != "program":
+                lib.bt_last_error.restype = ctypes.c_char_p
+            for entry in _CALLS:
                 if hasattr(lib, entry):
-                    getattr(lib, entry).argtypes = types
+                    getattr(lib, entry).argtypes = [_c_ptr, _c_ptr]
             _modules[name] = lib
         return lib
 
@@ -166,6 +184,87 @@ def _module(name):
 def _check(lib, code):
     if code != 0:
         raise KernelError(lib.bt_last_error().decode())
+
+
+_recorder = [None]      # the Program that kernels are being written into instead of being launched
+
+
+def _launch(lib, name, call):
+    """Calls a kernel's structure form now, or, while a launch list is being recorded, keeps the
+    pair for later."""
+    program = _recorder[0]
+    if program is not None:
+        program.add(lib, name, call)
+        return
+    _check(lib, getattr(lib, name)(_stream(), ctypes.byref(call)))
+
+
+class Program:
+    """A launch list: the kernel calls of one step, in order, each as (entry point, argument
+    structure).  ``run`` hands the whole list to one C++ loop (csrc/program.cpp), so a step costs
+    the host one call from Python plus the launches themselves.
+
+        program = Program()
+        with program.recording():
+            model.forward(step, cache)        # nothing is launched; every kernels.library call is kept
+        program.run()                         # launches them all, now and as often as wanted
+
+    What the list holds is only addresses and sizes: it stays valid as long as every buffer, table
+    and weight it names stays where it is, and gives the same results as calling the kernels one
+    by one, bit for bit (they are the same calls)."""
+
+    def __init__(self):
+        self.calls = []             # (module, entry point name, structure); the structures are kept alive here
+        self._entries = None
+
+    def add(self, lib, name, call):
+        self.calls.append((lib, name, call))
+        self._entries = None
+
+    def recording(self):
+        return _Recording(self)
+
+    def __len__(self):
+        return len(self.calls)
+
+    def _freeze(self):
+        entries = (LaunchEntry * max(len(self.calls), 1))()
+        for i, (lib, name, call) in enumerate(self.calls):
+            entries[i].call = ctypes.cast(getattr(lib, name), _c_ptr).value
+            entries[i].args = ctypes.addressof(call)
+        self._entries = entries
+
+    def run(self):
+        """Launches every call of the list on the current stream."""
+        if self._entries is None:
+            self._freeze()
+        runner = _module("program")
+        failed = _c_int(-1)
+        code = runner.bt_program_run(_c_ptr(_stream()), self._entries, _c_int(len(self.calls)), ctypes.byref(failed))
+        if code != 0:
+            lib, name, _ = self.calls[failed.value]
+            raise KernelError(f"{lib.bt_last_error().decode()} (call {failed.value} of {len(self.calls)}, {name})")
+
+
+class _Recording:
+    def __init__(self, program):
+        self.program = program
+
+    def __enter__(self):
+        if _recorder[0] is not None:
+            raise RuntimeError("a launch list is already being recorded")
+        _recorder[0] = self.program
+        return self.program
+
+    def __exit__(self, *exc):
+        _recorder[0] = None
+        return False
+
+
+def recording():
+    """True while kernel calls are being kept in a launch list instead of being launched: a part
+    that does anything but call this module's kernels cannot be recorded."""
+    return _recorder[0] is not None
 
 
 _held_stream = [None]
@@ -209,7 +308,7 @@ def require_gpu():
 
 def prepare(dtype, head_dims=()):
     """Builds and loads what a model of this dtype and these head sizes needs."""
-    names = ["core", "gemm_mfma"]
+    names = ["core", "gemm_mfma", "program"]
     if dtype == torch.bfloat16:
         if os.environ.get(PRODUCTS_ENV, "") != "own":
             names.append("gemm_library")
@@ -331,10 +430,9 @@ def epilogue_qkv(q_out, n_q, n_kv, kv_view, tok_seq, tok_pos, bias=None):
 
 def embed(ids, positions, table, position_table, out):
     """out[t] = table[ids[t]] (+ position_table[positions[t]]); out is the float32 stream."""
-    lib = _module("core")
-    _check(lib, lib.bt_embed(_stream(), DTYPE_CODES[table.dtype], ids.data_ptr(),
-                             _ptr(positions), table.data_ptr(), _ptr(position_table),
-                             out.data_ptr(), ids.numel(), table.shape[1]))
+    _launch(_module("core"), "bt_embed_call",
+            EmbedCall(dtype=DTYPE_CODES[table.dtype], tokens=ids.numel(), width=table.shape[1], ids=ids.data_ptr(),
+                      pos=_ptr(positions), table=table.data_ptr(), positions=_ptr(position_table), out=out.data_ptr()))
 
 
 def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None, rows=None,
@@ -353,11 +451,11 @@ def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None,
     if delta is None and bias is None:
         write_back = False      # nothing is added: the stream already holds what would be written
     out_dtype = DTYPE_CODES[out.dtype] if out is not None else FLOAT32
-    _check(lib, lib.bt_add_norm(
-        _stream(), out_dtype, x.data_ptr(), _ptr(delta), n_delta,
-        stride, _ptr(bias), _ptr(gamma), _ptr(beta), eps,
-        NORM_KINDS[kind], out.data_ptr() if out is not None else None, _ptr(rows), n_rows, width,
-        1 if write_back else 0, _out_rows(out)))
+    _launch(lib, "bt_add_norm_call",
+            AddNormCall(out_dtype=out_dtype, n_delta=n_delta, kind=NORM_KINDS[kind], n_rows=n_rows, width=width,
+                        write_back=1 if write_back else 0, out_rows=_out_rows(out), eps=eps, x=x.data_ptr(),
+                        delta=_ptr(delta), delta_stride=stride, bias=_ptr(bias), gamma=_ptr(gamma), beta=_ptr(beta),
+                        out=out.data_ptr() if out is not None else None, rows=_ptr(rows)))
 
 
 def pack_columns(w, columns):
@@ -449,10 +547,10 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
             raise KernelError(f"gemm: rows to be normalised [{m},{k}] go with bfloat16 weights [{n},{k}] on the skinny kernel only")
         operand = NormOperand(x=a.x.data_ptr(), ldx=a.x.stride(0), gamma=a.gamma.data_ptr(), beta=_ptr(a.beta),
                               eps=a.eps, kind=NORM_KINDS[a.kind])
-        lib = _module("gemm_mfma")
         weights, columns = (packed[0].data_ptr(), packed[1]) if packed is not None else (w.data_ptr(), 0)
-        _check(lib, lib.bt_gemm_skinny(_stream(), BFLOAT16, None, 0, weights, m, n, k, epilogue, splits,
-                                       variant, operand, columns, 0))
+        _launch(_module("gemm_mfma"), "bt_gemm_skinny_call",
+                GemmCall(dtype=BFLOAT16, M=m, N=n, K=k, splits=splits, variant=variant, packed_columns=columns,
+                         has_norm=1, W=weights, epi=epilogue, norm=operand))
         return
     if w.shape[1] != k or a.stride(1) != 1 or not w.is_contiguous() or a.dtype != w.dtype:
         raise KernelError(f"gemm: operands [{m},{k}] {a.dtype} and [{n},{w.shape[1]}] {w.dtype} do not fit")
@@ -465,28 +563,15 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
         elif dtype == FLOAT32:
             impl = "tile"
         else:
-            shape = (m, n, k, int(epilogue.mode), bool(epilogue.bias))
             impl = "library" if splits == 1 and _library_takes(epilogue) and library_products() \
-                and shape not in _library_refused else "tile"
-            if impl == "library":
-                try:
-                    gemm(a, w, epilogue, impl="library")
-                    return
-                except KernelError as refusal:      # the library has nothing for this shape: the tile kernel does
-                    if "no algorithm" not in str(refusal):
-                        raise
-                    _library_refused.add(shape)
-                    print(f"[burn_transformers_amd] {refusal}; this shape runs on the package's tile kernel",
-                          file=sys.stderr, flush=True)
-                    impl = "tile"
-    args = (a.data_ptr(), a.stride(0), w.data_ptr(), m, n, k, epilogue)
+                and _library_has_algorithm(a.stride(0), m, n, k, epilogue) else "tile"
+    call = GemmCall(dtype=dtype, M=m, N=n, K=k, splits=splits, variant=variant, A=a.data_ptr(), lda=a.stride(0),
+                    W=w.data_ptr(), epi=epilogue)
     if impl == "plain":
         if splits != 1:
             raise KernelError("gemm: the plain kernel does not split K")
-        lib = _module("core")
-        _check(lib, lib.bt_gemm_plain(_stream(), dtype, *args))
-        return
-    if impl == "library":
+        _launch(_module("core"), "bt_gemm_plain_call", call)
+    elif impl == "library":
         if dtype != BFLOAT16 or epilogue.out_rows:
             raise KernelError("gemm: the library product takes bfloat16 only and writes row-major results")
         lib = _library_state["lib"] or library_products()
@@ -494,15 +579,33 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
             raise KernelError("gemm: the vendor's GEMM library is not available")
         if splits != 1:
             raise KernelError("gemm: the library product does not split K")
-        _check(lib, lib.bt_gemm_library_bf16(_stream(), *args))
-        return
-    lib = _module("gemm_mfma")
-    if impl == "tile":
-        _check(lib, lib.bt_gemm_tile(_stream(), dtype, *args, splits, variant))
+        _launch(lib, "bt_gemm_library_call", call)
+    elif impl == "tile":
+        _launch(_module("gemm_mfma"), "bt_gemm_tile_call", call)
     else:
+        call.a_rows = a_rows
         if packed is not None:          # (only here: the other kernels read the plain matrix)
-            args = (a.data_ptr(), a.stride(0), packed[0].data_ptr(), m, n, k, epilogue)
-        _check(lib, lib.bt_gemm_skinny(_stream(), dtype, *args, splits, variant, None, packed[1] if packed is not None else 0, a_rows))
+            call.W, call.packed_columns = packed[0].data_ptr(), packed[1]
+        _launch(_module("gemm_mfma"), "bt_gemm_skinny_call", call)
+
+
+def _library_has_algorithm(lda, m, n, k, epilogue):
+    """Whether the vendor's library has an algorithm for this product (asked without running
+    anything; the library keeps what it found).  A shape it has none for is remembered and runs on
+    the package's tile kernel, with a line on stderr the first time."""
+    shape = (m, n, k, int(epilogue.mode), bool(epilogue.bias))
+    if shape in _library_refused:
+        return False
+    lib = _library_state["lib"]
+    if lib.bt_gemm_library_plan(_c_i64(lda), _c_int(m), _c_int(n), _c_int(k), ctypes.byref(epilogue)) == 0:
+        return True
+    refusal = lib.bt_last_error().decode()
+    if "no algorithm" not in refusal:
+        raise KernelError(refusal)
+    _library_refused.add(shape)
+    print(f"[burn_transformers_amd] {refusal}; this shape runs on the package's tile kernel",
+          file=sys.stderr, flush=True)
+    return False
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
@@ -534,30 +637,27 @@ def attention(args, dtype, decode, impl="auto"):
             impl = "mfma"
         else:
             impl = "tiled" if args.kv.head_dim <= 128 and args.kv.head_dim % 16 == 0 and args.ldq % 4 == 0 else "plain"
+    call = AttentionCall(dtype=code, args=args)
     if impl == "plain":
-        lib = _module("core")
-        _check(lib, lib.bt_attention_plain(_stream(), code, args))
+        _launch(_module("core"), "bt_attention_plain_call", call)
         return
     if impl == "tiled":
         if code != FLOAT32:
             raise KernelError("attention: the tiled kernel takes float32 only")
-        lib = _module("attention_f32")
-        _check(lib, lib.bt_attention_f32(_stream(), args))
+        _launch(_module("attention_f32"), "bt_attention_f32_call", call)
         return
     if code != BFLOAT16:
         raise KernelError("attention: the MFMA kernels take bfloat16 only")
-    lib = _module(f"attention_bf16_hd{args.kv.head_dim}")
-    fn = lib.bt_attention_decode_bf16 if decode else lib.bt_attention_prefill_bf16
-    _check(lib, fn(_stream(), args))
+    _launch(_module(f"attention_bf16_hd{args.kv.head_dim}"),
+            "bt_attention_decode_bf16_call" if decode else "bt_attention_prefill_bf16_call", call)
 
 
 def kv_copy(k_rows, v_rows, tok_seq, tok_pos, kv_view, to_cache):
     """Copies [tokens, kv_heads * head_dim] rows into the paged cache, or back out of it."""
-    lib = _module("core")
-    _check(lib, lib.bt_kv_copy(_stream(), DTYPE_CODES[k_rows.dtype], k_rows.data_ptr(),
-                               v_rows.data_ptr(), k_rows.stride(0), tok_seq.data_ptr(),
-                               tok_pos.data_ptr(), kv_view, k_rows.shape[0],
-                               1 if to_cache else 0))
+    _launch(_module("core"), "bt_kv_copy_call",
+            KvCopyCall(dtype=DTYPE_CODES[k_rows.dtype], tokens=k_rows.shape[0], to_cache=1 if to_cache else 0,
+                       k_rows=k_rows.data_ptr(), v_rows=v_rows.data_ptr(), ld=k_rows.stride(0),
+                       tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), kv=kv_view))
 
 
 _sample_workspaces = {}

@@ -35,6 +35,7 @@ RUN_BYTES = 128 << 10
 @register("mixer", "attention")
 class CausalSelfAttention(Mixer):
     takes_deferred_norm = True
+    only_launches_kernels = True
 
     def __init__(self, params, tensors):
         super().__init__(params, tensors)

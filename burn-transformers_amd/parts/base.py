@@ -93,6 +93,14 @@ class Memory:
 
 
 class Part:
+    # True for a part whose step does nothing but call kernels of ``kernels.library`` with
+    # arguments that depend only on the step's shape and on addresses that stay where they are
+    # (weights, the step's workspaces and tables): the engine then keeps a step's calls as a launch
+    # list and walks it in C++ (``kernels.library.Program``).  A part that computes with torch,
+    # reads the step's host tables or allocates in its step leaves this False, and every step of a
+    # model that holds such a part is issued from Python, call by call.
+    only_launches_kernels = False
+
     def __init__(self, params, tensors):
         self.params, self.tensors = params, tensors
 
@@ -176,9 +184,14 @@ class Block:
     the engine asks the block, not the names, what it needs."""
 
     ROLES = {}
+    only_launches_kernels = False       # as for a part: True if ``forward`` only calls its parts and the stream
 
     def __init__(self, parts):
         self.parts = parts
+
+    def recordable(self):
+        """Whether a step of this block can be kept as a launch list."""
+        return self.only_launches_kernels and all(part.only_launches_kernels for part in self.parts.values())
 
     def mixers(self):
         """The parts of this block that mix tokens (they say what the cache has to keep and which

@@ -17,6 +17,7 @@ MIXER_FOLD_ROWS = 4
 @register("block", "pre_norm")
 class PreNormBlock(Block):
     ROLES = {"mixer_norm": "norm", "mixer": "mixer", "ff_norm": "norm", "ff": "feed_forward"}
+    only_launches_kernels = True
 
     def forward(self, stream, step, memory):
         parts = self.parts

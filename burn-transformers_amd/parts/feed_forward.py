@@ -20,6 +20,7 @@ from .registry import register
 @register("feed_forward", "dense")
 class DenseFeedForward(FeedForward):
     takes_deferred_norm = True
+    only_launches_kernels = True
 
     def __init__(self, params, tensors):
         super().__init__(params, tensors)

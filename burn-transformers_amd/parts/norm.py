@@ -14,6 +14,7 @@ from .registry import register
 
 class _KernelNorm(Norm):
     KIND = None
+    only_launches_kernels = True
 
     def __init__(self, params, tensors):
         super().__init__(params, tensors)

@@ -12,6 +12,8 @@ from .registry import register
 
 @register("embedding", "learned_positions")
 class LearnedPositionEmbedding(Embedding):
+    only_launches_kernels = True
+
     def __init__(self, params, tensors):
         super().__init__(params, tensors)
         self.width, self.vocab_size = params["width"], params["vocab_size"]
@@ -29,6 +31,8 @@ class LearnedPositionEmbedding(Embedding):
 
 @register("embedding", "token_only")
 class TokenEmbedding(Embedding):
+    only_launches_kernels = True
+
     def __init__(self, params, tensors):
         super().__init__(params, tensors)
         self.width, self.vocab_size = params["width"], params["vocab_size"]

@@ -8,6 +8,7 @@ from .registry import register
 
 @register("readout", "linear_readout")
 class LinearReadout(Readout):
+    only_launches_kernels = True
     takes_deferred_norm = True       # the rows are only handed to ``gemm``: the final norm may leave them chunk-major
 
     def __init__(self, params, tensors):

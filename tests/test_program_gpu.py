@@ -1,0 +1,137 @@
+"""Launch lists: a step's kernel calls kept as (entry point, structure) pairs and walked in C++.
+
+A list is recorded from the same parts that issue kernels one by one, so both ways run the same
+kernels with the same arguments: every result here is compared bit for bit."""
+
+import time
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import burn_transformers_amd as bt  # noqa: E402
+from burn_transformers_amd.kernels import library as K  # noqa: E402
+from model_helpers import model_folder, plain_logits, prompts_for, tolerance  # noqa: E402
+
+_models = {}
+
+
+def model_for(name, dtype):
+    if (name, dtype) not in _models:
+        folder, _, _ = model_folder(name)
+        _models[(name, dtype)] = bt.load_model(folder, dtype=dtype, device="cuda:0")
+    return _models[(name, dtype)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "BW", "C"])
+def test_steps_from_launch_lists_equal_steps_issued_one_by_one(name, dtype):
+    """A random schedule of prompts, chunks and single tokens on two engines of one model, one
+    walking launch lists and one calling every kernel from Python; no graphs in either."""
+    model = model_for(name, dtype)
+    assert model.recordable
+    listed = bt.Engine(model, max_tokens=64 * 12, graphs=False)
+    direct = bt.Engine(model, max_tokens=64 * 12, graphs=False, programs=False)
+    assert listed.use_programs and not direct.use_programs
+    gen = torch.Generator().manual_seed(3)
+    limit = model.max_positions
+    requests = prompts_for(name, [limit - 3, 40, 70, 9], seed=81)
+    slots = [(listed.open(), direct.open()) for _ in requests]
+    fed = [0] * len(requests)
+    shapes = set()
+    for turn in range(40):
+        live = [i for i in range(len(requests)) if fed[i] < len(requests[i])]
+        if not live:
+            break
+        chosen = [i for i in live if int(torch.randint(0, 3, (1,), generator=gen)) > 0] or live[:1]
+        counts = [1 if turn % 3 == 2 else int(torch.randint(1, 24, (1,), generator=gen)) for _ in chosen]
+        entries_l = [(slots[i][0], requests[i][fed[i]:fed[i] + c]) for i, c in zip(chosen, counts)]
+        entries_d = [(slots[i][1], requests[i][fed[i]:fed[i] + c]) for i, c in zip(chosen, counts)]
+        want = [list(range(len(e[1]))) for e in entries_l]
+        a = listed.step(entries_l, want).clone()
+        b = direct.step(entries_d, want).clone()
+        assert torch.equal(a, b), f"turn {turn}"
+        shapes.add(tuple(len(e[1]) for e in entries_l))
+        for i, e in zip(chosen, entries_l):
+            fed[i] += len(e[1])
+    assert listed.program_runs == listed.steps_run and direct.program_runs == 0
+    # and against the plain implementation, through the list that was used most recently
+    ids = requests[1]
+    slot = listed.open()
+    logits = listed.step([(slot, ids)], want=[list(range(len(ids)))])
+    want = plain_logits(name, ids)
+    assert float((logits.cpu().double() - want).abs().max()) <= tolerance(dtype, want)
+    listed.reset()
+    direct.reset()
+
+
+def test_a_repeated_shape_reuses_its_list_and_a_grown_workspace_makes_lists_stale():
+    model = model_for("A", "bfloat16")
+    engine = bt.Engine(model, max_tokens=64 * 40, graphs=False)
+    ids = prompts_for("A", [20], seed=82)[0]
+    want = plain_logits("A", ids)
+    outs = []
+    for _ in range(3):
+        slot = engine.open()
+        outs.append(engine.step([(slot, ids)], want=[list(range(20))]).clone())
+        engine.close(slot)
+    assert len(engine._programs) == 1 and torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+    # a much larger step makes the workspaces grow: the old list names addresses that are gone
+    many = prompts_for("A", [120] * 16, seed=83)
+    slots = [engine.open() for _ in many]
+    engine.step(list(zip(slots, many)))
+    for slot in slots:
+        engine.close(slot)
+    slot = engine.open()
+    again = engine.step([(slot, ids)], want=[list(range(20))]).clone()
+    assert torch.equal(again, outs[0])
+    assert float((again.cpu().double() - want).abs().max()) <= tolerance("bfloat16", want)
+
+
+def test_a_call_that_refuses_names_itself_and_the_step_changes_nothing():
+    """The walk stops at the call that refuses; the message is that kernel's own."""
+    model = model_for("A", "float32")
+    engine = bt.Engine(model, max_tokens=256, graphs=False)
+    slot = engine.open()
+    ids = prompts_for("A", [30], seed=84)[0]
+    engine.step([(slot, ids[:10])])
+    program, _ = next(iter(engine._programs.values()))
+    # break one call of the recorded list: a product of rows that no kernel takes
+    index = next(i for i, (_, name, _) in enumerate(program.calls) if name == "bt_gemm_skinny_call")
+    call = program.calls[index][2]
+    rows = call.M
+    call.M = 65
+    slot2 = engine.open()
+    before = (engine.length(slot2), list(engine.cache.blocks(slot2)))
+    with pytest.raises(K.KernelError, match=r"gemm_skinny: 65 rows, at most 64 \(call \d+ of \d+, bt_gemm_skinny_call\)"):
+        engine.step([(slot2, ids[:10])])
+    assert (engine.length(slot2), list(engine.cache.blocks(slot2))) == before
+    engine.cache.ledger.check()
+    call.M = rows
+    logits = engine.step([(slot2, ids[:10])])
+    want = plain_logits("A", ids[:10])[-1:]
+    assert float((logits.cpu().double() - want).abs().max()) <= tolerance("float32", want)
+
+
+def test_host_time_of_a_listed_step_is_a_fraction_of_the_direct_one():
+    """What the list is for: the host's share of a step.  Measured without waiting for the GPU
+    (the calls only queue work): the same steps issued from Python cost several times more."""
+    model = model_for("BW", "bfloat16")
+    ids = prompts_for("BW", [64], seed=85)[0]
+    seconds = {}
+    for programs in (True, False):
+        engine = bt.Engine(model, max_tokens=64 * 4, graphs=False, programs=programs)
+        slot = engine.open()
+        engine.step([(slot, ids)])
+        engine.truncate(slot, 0)
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        for _ in range(20):
+            engine.step([(slot, ids)])
+            engine.truncate(slot, 0)
+        seconds[programs] = (time.perf_counter() - started) / 20
+        torch.cuda.synchronize()
+    print(f"host time of a 64-token step of a 3-layer model: {seconds[True] * 1e6:.0f} us from a launch list, "
+          f"{seconds[False] * 1e6:.0f} us call by call")
+    assert seconds[True] < 0.7 * seconds[False]

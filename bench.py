@@ -1,33 +1,58 @@
-"""Throughput of GPT-2 XL-sized generation on one MI355X.
+"""Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
+                    [--repetitions 10] [--workload xl|small|medium] [--no-points] [--no-kernels]
 
-With no flags, 16 untimed and 495 timed steps take the sequences from 512 to 1,024 tokens.
+The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
+sequences, prefilled with 512 synthetic tokens each, is decoded towards 1,024.  A step is one
+decode step of the whole batch: the engine's step function followed by greedy selection and the
+readback of the chosen ids, exactly what the generation loop runs.  With no flags, 16 untimed and
+495 timed steps take the sequences from 512 to 1,024 tokens.
 
-A step is one decode step of the whole batch: the engine's step function followed by greedy
-selection and the readback of the chosen ids, exactly what the generation loop runs.  The
-default run has the layer sizes of GPT-2 XL with random weights, a batch of 8 sequences that
-were prefilled with 512 synthetic tokens each and are decoded to 1,024.  One JSON line
-is printed:
-  value      decoded tokens per second over the K timed steps
-  prefill    one step of 2 x 1,024 prompt tokens: tokens/s, ms, fraction of the MFMA peak
-  roofline   bytes a decode step has to read (every weight once + the live cache) / its time,
-             against 8 TB/s
-  points     decoded tokens per second at batch 1 and 64
+The protocol is the reference's (BENCHMARKS.md:71-87, tests/support/causal_decode_benchmark.rs:
+1-31): 3 warm-up repetitions and 10 measured ones, every repetition on fresh sequences (new slots,
+a new prefill), the device synchronised at both ends of the timed steps, forced length (no end
+token), real tokens only; the median repetition is the value, the fastest and slowest are given.
+
+One JSON line is printed:
+  value       decoded tokens per second over the K timed steps of the median repetition
+  spread      milliseconds per step of the fastest, median and slowest repetition
+  prefill     one step of 2 x 1,024 prompt tokens: tokens/s, ms, fraction of the MFMA peak;
+              `own` is the same step with every product on this package's kernels (the default
+              hands products of more than 64 rows to hipBLASLt, as the reference hands its
+              products to its backend's library)
+  roofline    bytes a decode step has to read (every weight once + the live cache) / its time,
+              against 8 TB/s
+  points      decoded tokens per second at batch 1 and 64
+  kernels     for the decode step and for the prefill step, each class of kernel on its own: the
+              step's launch list is cut into classes (same kernel, same shape), each class's calls
+              (one per layer, every layer's own weights) are replayed alone from a HIP graph and
+              timed with events; per call: microseconds and the fraction of the HBM roofline
+              (decode) or of the MFMA peak (prefill)
+
+``--workload small`` and ``--workload medium`` run the other two measured workloads through the
+generation loop: GPT-2 small sizes in float32, 16 prompts of 1 to 1,000 tokens decoded greedily to
+1,024 tokens each; GPT-2 medium sizes, 64 prompts of 64 to 768 tokens prefilled in chunks of 256
+and sampled at temperature 1 to 1,024 tokens each.  Their value is generated tokens per second.
 """
 
 import argparse
 import json
+import statistics
 import sys
 import time
 
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+ELEMENT_BYTES = {"bf16": 2, "fp32": 4}
 
 XL = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 48, "n_embd": 1600, "n_head": 25,
       "n_inner": 6400, "vocab_size": 50257, "n_positions": 1024, "activation_function": "gelu_new",
       "layer_norm_epsilon": 1e-5}
+SMALL = dict(XL, n_layer=12, n_embd=768, n_head=12, n_inner=3072)
+MEDIUM = dict(XL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
 PROMPT_LEN, CONTEXT_LEN, PREFILL_SEQS, PREFILL_LEN = 512, 1024, 2, 1024
+WARMUP_REPETITIONS = 3
 
 
 def build_model(config, dtype):
@@ -53,14 +78,13 @@ def synthetic_prompts(batch, length, vocab, seed):
     return torch.randint(0, vocab, (batch, length), generator=gen).tolist()
 
 
-def decode_run(engine, batch, warmup, steps, vocab):
-    """(seconds for `steps` decode steps, mean context length over them)."""
+def decode_repetition(engine, batch, warmup, steps, vocab, seed):
+    """One repetition on fresh sequences: (seconds of the timed steps, first context length)."""
     import torch
 
     import burn_transformers_amd as bt
     from burn_transformers_amd.sampling.sampler import Sampler
-    steps = min(steps, CONTEXT_LEN - PROMPT_LEN - warmup - 1)
-    prompts = synthetic_prompts(batch, PROMPT_LEN, vocab, seed=batch)
+    prompts = synthetic_prompts(batch, PROMPT_LEN, vocab, seed=seed)
     slots = [engine.open() for _ in prompts]
     sampler = Sampler(bt.GenerationConfig(), batch, engine.device)
     rows = list(range(batch))
@@ -84,18 +108,30 @@ def decode_run(engine, batch, warmup, steps, vocab):
         ids = one_step(ids)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
-    mean_context = first_context + (steps + 1) / 2.0     # keys each step's query reads, itself included
     for slot in slots:
         engine.close(slot)
-    return elapsed, steps, mean_context
+    return elapsed, first_context
 
 
-def prefill_run(engine, vocab, repeats=5):
-    """Median seconds of one step of PREFILL_SEQS x PREFILL_LEN prompt tokens."""
+def decode_run(engine, batch, warmup, steps, vocab, repetitions, warmup_repetitions=WARMUP_REPETITIONS):
+    """(sorted seconds of the measured repetitions, steps, mean context length over the timed steps)."""
+    steps = max(1, min(steps, CONTEXT_LEN - PROMPT_LEN - warmup - 1))
+    for r in range(warmup_repetitions):          # short: they are there for graphs, clocks and caches
+        decode_repetition(engine, batch, warmup, min(steps, 24), vocab, seed=1000 + r)
+    times, first_context = [], PROMPT_LEN
+    for r in range(repetitions):
+        elapsed, first_context = decode_repetition(engine, batch, warmup, steps, vocab, seed=batch * 100 + r)
+        times.append(elapsed)
+    mean_context = first_context + (steps + 1) / 2.0     # keys each step's query reads, itself included
+    return sorted(times), steps, mean_context
+
+
+def prefill_run(engine, vocab, repetitions):
+    """Sorted seconds of one step of PREFILL_SEQS x PREFILL_LEN prompt tokens on fresh sequences."""
     import torch
-    prompts = synthetic_prompts(PREFILL_SEQS, PREFILL_LEN, vocab, seed=99)
     times = []
-    for _ in range(repeats + 1):
+    for r in range(WARMUP_REPETITIONS + repetitions):
+        prompts = synthetic_prompts(PREFILL_SEQS, PREFILL_LEN, vocab, seed=99 + r)
         slots = [engine.open() for _ in prompts]
         torch.cuda.synchronize()
         started = time.perf_counter()
@@ -104,20 +140,243 @@ def prefill_run(engine, vocab, repeats=5):
         times.append(time.perf_counter() - started)
         for slot in slots:
             engine.close(slot)
-    times = sorted(times[1:])
-    return times[len(times) // 2]
+    return sorted(times[WARMUP_REPETITIONS:])
 
 
-def model_bytes_and_flops(config, layers):
+def model_bytes_and_flops(config, layers, dtype):
+    """(bytes of every weight a step reads, bytes of keys and values per cached token, flops of the
+    prefill step): matrices and the cache in the element type of the run, vectors in float32."""
     d, m, v = config["n_embd"], config["n_inner"], config["vocab_size"]
+    element = ELEMENT_BYTES[dtype]
     per_layer = 3 * d * d + d * d + 2 * d * m           # matrix elements
     vectors = 3 * d + d + m + d + 4 * d
-    weight_bytes = 2 * (layers * per_layer + v * d) + 4 * (layers * vectors + 2 * d)
-    kv_bytes_per_token = 2 * layers * d * 2
+    weight_bytes = element * (layers * per_layer + v * d) + 4 * (layers * vectors + 2 * d)
+    kv_bytes_per_token = 2 * layers * d * element
     dense = 2.0 * PREFILL_SEQS * PREFILL_LEN * layers * per_layer
     attention = layers * PREFILL_SEQS * 2.0 * d * PREFILL_LEN * (PREFILL_LEN + 1)
     readout = 2.0 * PREFILL_SEQS * d * v
     return weight_bytes, kv_bytes_per_token, dense + attention + readout
+
+
+# --- each class of kernel on its own -----------------------------------------------------------
+
+def _class_of(name, call):
+    """(label, bytes a call has to read, flops it does) of one recorded kernel call."""
+    short = name[len("bt_"):-len("_call")]
+    if short.startswith("gemm"):
+        element = 4 if call.dtype == 0 else 2
+        weights = call.N * call.K * element
+        rows = call.M * call.K * (4 if call.has_norm else element)
+        return f"{short} {call.M}x{call.N}x{call.K}", weights + rows, 2.0 * call.M * call.N * call.K
+    if short.startswith("attention"):
+        return f"{short} {call.args.n_tokens}tok", None, None       # filled in by the caller, who knows the contexts
+    if short == "add_norm":
+        return f"add_norm {call.n_rows}x{call.width}", (call.n_delta + 2) * call.n_rows * call.width * 4, 0.0
+    if short == "embed":
+        return f"embed {call.tokens}x{call.width}", call.tokens * call.width * 6, 0.0
+    if short == "kv_copy":
+        return f"kv_copy {call.tokens}tok", call.tokens * call.kv.kv_heads * call.kv.head_dim * 8, 0.0
+    return short, 0, 0.0
+
+
+def kernel_classes(engine, entries, attention_bytes, attention_flops, peak_flops, replays=20):
+    """Runs one step of ``entries`` to get its launch list, then replays each class of calls alone
+    from a HIP graph.  Returns {label: {"n": calls a step, "us": per call, "hbm": fraction of the
+    HBM roofline, "mfma": fraction of the MFMA peak}}."""
+    import torch
+    from burn_transformers_amd.kernels import library as K
+    if not engine.use_programs:
+        return {}
+    before = set(engine._programs)
+    graphs, engine.use_graphs = engine.use_graphs, False
+    try:
+        engine.step(entries)
+        torch.cuda.synchronize()
+    finally:
+        engine.use_graphs = graphs
+    fresh = [key for key in engine._programs if key not in before] or list(engine._programs)[-1:]
+    program = engine._programs[fresh[-1]][0]
+    classes = {}
+    for lib, name, call in program.calls:
+        label, nbytes, flops = _class_of(name, call)
+        if nbytes is None:
+            nbytes, flops = attention_bytes, attention_flops
+        classes.setdefault(label, []).append((lib, name, call, nbytes, flops))
+    out = {}
+    for label, calls in classes.items():
+        part = K.Program()
+        repeat = -(-8 // len(calls))                 # a class of one or two calls is run eight times over:
+        for _ in range(repeat):                      # a graph of a single kernel measures the graph's launch
+            for lib, name, call, _, _ in calls:
+                part.add(lib, name, call)
+        part.run()                                   # once outside a graph (first-use set-up of a kernel)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            part.run()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        times = []
+        for _ in range(replays):
+            begin.record()
+            graph.replay()
+            end.record()
+            end.synchronize()
+            times.append(begin.elapsed_time(end) * 1e-3 / len(part))
+        seconds = statistics.median(times)
+        nbytes, flops = calls[0][3], calls[0][4]
+        out[label] = {"n": len(calls), "us": round(seconds * 1e6, 2),
+                      "hbm": round(nbytes / seconds / 1e9 / PEAK_HBM_GBS, 3),
+                      "mfma": round(flops / seconds / peak_flops, 3)}
+    return out
+
+
+def decode_kernels(engine, batch, vocab, config, dtype, context):
+    """Classes of a decode step of ``batch`` sequences that hold ``context`` tokens each."""
+    prompts = synthetic_prompts(batch, context - 1, vocab, seed=7)
+    slots = [engine.open() for _ in prompts]
+    for begin in range(0, batch, 8):
+        engine.step([(slots[i], prompts[i]) for i in range(begin, min(begin + 8, batch))])
+    d = config["n_embd"]
+    kv_bytes = batch * context * 2 * d * ELEMENT_BYTES[dtype]        # one layer's keys and values of the live context
+    try:
+        return kernel_classes(engine, [(slot, [5]) for slot in slots], kv_bytes, 4.0 * batch * context * d,
+                              PEAK_FLOPS[dtype])
+    finally:
+        for slot in slots:
+            engine.close(slot)
+
+
+def prefill_kernels(engine, vocab, config, dtype):
+    prompts = synthetic_prompts(PREFILL_SEQS, PREFILL_LEN, vocab, seed=8)
+    slots = [engine.open() for _ in prompts]
+    d = config["n_embd"]
+    tokens = PREFILL_SEQS * PREFILL_LEN
+    try:
+        return kernel_classes(engine, list(zip(slots, prompts)), 4 * tokens * d * ELEMENT_BYTES[dtype],
+                              PREFILL_SEQS * 2.0 * d * PREFILL_LEN * (PREFILL_LEN + 1), PEAK_FLOPS[dtype], replays=10)
+    finally:
+        for slot in slots:
+            engine.close(slot)
+
+
+# --- the workloads -----------------------------------------------------------------------------
+
+def run_xl(args):
+    import torch  # noqa: F401
+
+    import burn_transformers_amd as bt
+    from burn_transformers_amd.kernels import library as K
+
+    config = dict(XL, n_layer=args.layers)
+    model = build_model(config, args.dtype)
+    vocab = config["vocab_size"]
+    weight_bytes, kv_per_token, prefill_flops = model_bytes_and_flops(config, args.layers, args.dtype)
+    engine = bt.Engine(model, max_tokens=max(args.batch, 64) * CONTEXT_LEN)
+
+    times, steps, mean_context = decode_run(engine, args.batch, args.warmup, args.steps, vocab, args.repetitions)
+    median = statistics.median(times)
+    ms_per_step = 1000.0 * median / steps
+    value = args.batch * steps / median
+    step_bytes = weight_bytes + args.batch * mean_context * kv_per_token
+    achieved = step_bytes / (median / steps) / 1e9
+    final_context = PROMPT_LEN + args.warmup + steps + 1
+
+    prefill_times = prefill_run(engine, vocab, args.repetitions)
+    prefill_seconds = statistics.median(prefill_times)
+    prefill = {"value": round(PREFILL_SEQS * PREFILL_LEN / prefill_seconds, 1), "tokens": PREFILL_SEQS * PREFILL_LEN,
+               "ms": round(1000.0 * prefill_seconds, 3),
+               "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[args.dtype], 4),
+               "min_ms": round(1000.0 * prefill_times[0], 3), "max_ms": round(1000.0 * prefill_times[-1], 3),
+               "products": "hipBLASLt beyond 64 rows" if args.dtype == "bf16" and K.library_products() else "own kernels"}
+    kernels = {}
+    if not args.no_kernels:
+        kernels["decode"] = decode_kernels(engine, args.batch, vocab, config, args.dtype, int(mean_context))
+        kernels["prefill"] = prefill_kernels(engine, vocab, config, args.dtype)
+    if args.dtype == "bf16" and K.library_products() is not None:
+        # the same step with every product on this package's own kernels
+        held = dict(K._library_state)
+        K._library_state.update(tried=True, lib=None)
+        try:
+            own_engine = bt.Engine(model, max_tokens=PREFILL_SEQS * PREFILL_LEN)
+            own = statistics.median(prefill_run(own_engine, vocab, max(3, args.repetitions // 2)))
+            prefill["own"] = {"value": round(PREFILL_SEQS * PREFILL_LEN / own, 1), "ms": round(1000.0 * own, 3),
+                              "frac": round(prefill_flops / own / PEAK_FLOPS[args.dtype], 4)}
+            del own_engine
+        finally:
+            K._library_state.update(held)
+
+    points = {}
+    if not args.no_points:
+        for batch in (1, 64):
+            t, s, _ = decode_run(engine, batch, args.warmup, args.steps, vocab, max(3, args.repetitions // 2), 1)
+            points[f"decode_b{batch}"] = round(batch * s / statistics.median(t), 1)
+
+    return {
+        "metric": f"decode tok/s at batch {args.batch} (GPT-2 XL sizes, 512-token prompts decoded to "
+                  f"{final_context} tokens, median of {args.repetitions} repetitions)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic token ids, random weights",
+        "config": {"model": "gpt2-xl", "n_layer": args.layers, "n_layer_full": XL["n_layer"],
+                   "n_embd": config["n_embd"], "n_head": config["n_head"], "n_inner": config["n_inner"],
+                   "vocab_size": vocab, "n_positions": config["n_positions"], "global_batch": args.batch,
+                   "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LEN, "final_context": final_context,
+                   "mean_context": round(mean_context, 1), "parallelism": "single GPU", "decode_graphs": True,
+                   "repetitions": args.repetitions, "warmup_repetitions": WARMUP_REPETITIONS},
+        "spread": {"min_ms": round(1000.0 * times[0] / steps, 4), "median_ms": round(ms_per_step, 4),
+                   "max_ms": round(1000.0 * times[-1] / steps, 4)},
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+        "kernels": kernels,
+    }
+
+
+def run_generation(args):
+    """The small and the medium workload through the generation loop."""
+    import torch
+
+    import burn_transformers_amd as bt
+    if args.workload == "small":
+        config, count, low, high, chunk, dtype = SMALL, 16, 1, 1000, None, args.dtype or "fp32"
+        generation = bt.GenerationConfig(max_new_tokens=CONTEXT_LEN)
+        what = "GPT-2 small sizes, 16 prompts of 1 to 1,000 tokens decoded greedily to 1,024 tokens each"
+    else:
+        config, count, low, high, chunk, dtype = MEDIUM, 64, 64, 768, 256, args.dtype or "bf16"
+        generation = bt.GenerationConfig(max_new_tokens=CONTEXT_LEN, strategy="sample", temperature=1.0, seed=1)
+        what = ("GPT-2 medium sizes, 64 prompts of 64 to 768 tokens prefilled in chunks of 256 and sampled at "
+                "temperature 1 to 1,024 tokens each")
+    model = build_model(config, dtype)
+    engine = bt.Engine(model, max_tokens=count * CONTEXT_LEN)
+    gen = torch.Generator().manual_seed(17)
+    times, generated, prompt_tokens = [], 0, 0
+    repetitions = max(3, args.repetitions // 2)
+    for r in range(1 + repetitions):
+        lengths = torch.randint(low, high + 1, (count,), generator=gen).tolist()
+        prompts = [torch.randint(0, config["vocab_size"], (n,), generator=gen).tolist() for n in lengths]
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        out = bt.generate(engine, prompts, generation, prefill_chunk=chunk, total_length=CONTEXT_LEN)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        if r:                                        # the first repetition warms up
+            times.append((elapsed, sum(len(s.token_ids) for s in out), sum(lengths)))
+    times.sort(key=lambda t: t[1] / t[0])
+    elapsed, generated, prompt_tokens = times[len(times) // 2]
+    return {
+        "metric": f"generated tok/s ({what}; median of {repetitions} repetitions)",
+        "value": round(generated / elapsed, 1), "unit": "tokens/s", "n_gpus": 1, "steps": generated // count,
+        "warmup": 1, "ms_per_step": round(1000.0 * elapsed / max(1, CONTEXT_LEN - low), 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic token ids, random weights",
+        "config": {"model": "gpt2-" + args.workload, "n_layer": config["n_layer"], "n_embd": config["n_embd"],
+                   "n_head": config["n_head"], "n_inner": config["n_inner"], "vocab_size": config["vocab_size"],
+                   "n_positions": config["n_positions"], "global_batch": count, "prompt_len_min": low,
+                   "prompt_len_max": high, "seq_len": CONTEXT_LEN, "prefill_chunk": chunk or 0,
+                   "generated_tokens": generated, "prompt_tokens": prompt_tokens, "parallelism": "single GPU"},
+        "spread": {"min": round(times[0][1] / times[0][0], 1), "median": round(generated / elapsed, 1),
+                   "max": round(times[-1][1] / times[-1][0], 1)},
+    }
 
 
 def main():
@@ -127,53 +386,22 @@ def main():
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--layers", type=int, default=XL["n_layer"], help="fewer layers than the 48 of GPT-2 XL")
-    parser.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
+    parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
+    parser.add_argument("--workload", choices=["xl", "small", "medium"], default="xl")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    parser.add_argument("--no-kernels", action="store_true", help="skip the classes of kernels on their own")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this library")
         sys.exit(2)
-    import torch
-
-    import burn_transformers_amd as bt
-
-    config = dict(XL, n_layer=args.layers)
-    model = build_model(config, args.dtype)
-    vocab = config["vocab_size"]
-    weight_bytes, kv_per_token, prefill_flops = model_bytes_and_flops(config, args.layers)
-    engine = bt.Engine(model, max_tokens=max(args.batch, 64) * CONTEXT_LEN)
-
-    elapsed, steps, mean_context = decode_run(engine, args.batch, args.warmup, args.steps, vocab)
-    ms_per_step = 1000.0 * elapsed / steps
-    value = args.batch * steps / elapsed
-    step_bytes = weight_bytes + args.batch * mean_context * kv_per_token
-    achieved = step_bytes / (elapsed / steps) / 1e9
-
-    prefill_seconds = prefill_run(engine, vocab)
-    prefill = {"value": round(PREFILL_SEQS * PREFILL_LEN / prefill_seconds, 1), "tokens": PREFILL_SEQS * PREFILL_LEN,
-               "ms": round(1000.0 * prefill_seconds, 3),
-               "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[args.dtype], 4)}
-    points = {}
-    if not args.no_points:
-        for batch in (1, 64):
-            e, s, _ = decode_run(engine, batch, args.warmup, args.steps, vocab)
-            points[f"decode_b{batch}"] = round(batch * s / e, 1)
-
-    print(json.dumps({
-        "metric": f"decode tok/s at batch {args.batch} (GPT-2 XL sizes, 512-token prompts decoded to 1,024)",
-        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic token ids, random weights",
-        "config": {"model": "gpt2-xl", "n_layer": args.layers, "n_layer_full": XL["n_layer"],
-                   "n_embd": config["n_embd"], "n_head": config["n_head"], "n_inner": config["n_inner"],
-                   "vocab_size": vocab, "n_positions": config["n_positions"], "global_batch": args.batch,
-                   "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LEN, "mean_context": round(mean_context, 1),
-                   "parallelism": "single GPU", "decode_graphs": True},
-        "prefill": prefill,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
-        "points": points,
-    }))
+    if args.repetitions < 1:
+        parser.error("--repetitions must be at least 1")
+    if args.workload == "xl":
+        args.dtype = args.dtype or "bf16"
+        print(json.dumps(run_xl(args)))
+    else:
+        print(json.dumps(run_generation(args)))
 
 
 if __name__ == "__main__":

@@ -12,6 +12,7 @@
 
 #include <mutex>
 
+#define BT_EPILOGUE_ANY_HEAD_SIZE      // the plain product takes fused projections of any head size
 #include "host.h"
 #include "epilogue.h"
 #include "attention.h"

@@ -200,9 +200,12 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int N, int m, int n
     for (int i = 0; i < 4; ++i)
       if (i < count) v[i] += x[i];
     store4<float>(x, v, count, aligned);
+#ifdef BT_EPILOGUE_ANY_HEAD_SIZE
   } else if ((e.kv.head_dim & 3) != 0) {
-    // EPI_QKV with a head size that four columns do not divide (the plain product only): every
-    // column finds its own place among the queries, keys and values
+    // EPI_QKV with a head size that four columns do not divide: every column finds its own place
+    // among the queries, keys and values.  Compiled into the plain product only (it defines
+    // BT_EPILOGUE_ANY_HEAD_SIZE): the MFMA kernels refuse such head sizes, and in them this path
+    // would only cost registers (their tiles of 128 x 128 spilled with it, at a third of the speed).
     int seq = e.tok_seq[m], pos = e.tok_pos[m];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -220,6 +223,7 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int N, int m, int n
       if (!is_value) static_cast<T*>(e.kv.keys)[base + key_offset(e.kv.head_dim, pos, channel)] = from_float<T>(v[i]);
       else static_cast<T*>(e.kv.values)[base + value_offset(e.kv.head_dim, pos, channel)] = from_float<T>(v[i]);
     }
+#endif
   } else {  // EPI_QKV: head_dim (and with it n_q and n_kv) is a multiple of four, so the four columns share a head
     if (n0 < e.n_q) {
       store4<T>(static_cast<T*>(e.out) + (int64_t)m * e.ldo + n0, v, count, aligned);

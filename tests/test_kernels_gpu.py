@@ -85,6 +85,31 @@ def test_tile_gemm_forms_agree(variant, m, n, k):
                    variant=variant)
 
 
+def test_tile_product_keeps_its_speed_at_the_sizes_it_was_tuned_for():
+    """A guard against a change that makes the tile kernel spill its accumulators (an epilogue path
+    too many did, once: 75 -> 260 us): 2,048 x 4,800 x 1,600 in bfloat16 takes about 75 us (85 with
+    the activation), and the bound here is twice that."""
+    m, n, k = 2048, 4800, 1600
+    a = torch.randn(m, k, device=DEV).to(torch.bfloat16)
+    weights = [(torch.randn(n, k, device=DEV) * 0.02).to(torch.bfloat16) for _ in range(8)]
+    bias = torch.randn(n, device=DEV)
+    out = torch.empty(m, n, device=DEV, dtype=torch.bfloat16)
+    for act in (False, True):
+        make = (lambda: K.epilogue_act(out, "gelu_tanh", bias)) if act else (lambda: K.epilogue_store(out, bias))
+        K.gemm(a, weights[0], make(), impl="tile")
+        torch.cuda.synchronize()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best = float("inf")
+        for _ in range(3):
+            begin.record()
+            for w in weights:
+                K.gemm(a, w, make(), impl="tile")
+            end.record()
+            end.synchronize()
+            best = min(best, begin.elapsed_time(end) * 1e3 / len(weights))
+        assert best < 170.0, f"the tile product takes {best:.0f} us (activation epilogue: {act})"
+
+
 @pytest.mark.parametrize("m,n,k", [(65, 48, 72), (200, 300, 136), (300, 517, 1600), (2048, 1600, 320),
                                    (5000, 136, 72), (32768, 96, 64)])
 def test_vendor_library_products(m, n, k):

@@ -1,7 +1,7 @@
 """Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
-                    [--repetitions 10] [--workload xl|small|medium] [--no-points] [--no-kernels]
+                    [--repetitions 10] [--workload xl|small|medium|sweep] [--no-points] [--no-kernels]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
 sequences, prefilled with 512 synthetic tokens each, is decoded towards 1,024.  A step is one
@@ -34,6 +34,8 @@ One JSON line is printed:
 generation loop: GPT-2 small sizes in float32, 16 prompts of 1 to 1,000 tokens decoded greedily to
 1,024 tokens each; GPT-2 medium sizes, 64 prompts of 64 to 768 tokens prefilled in chunks of 256
 and sampled at temperature 1 to 1,024 tokens each.  Their value is generated tokens per second.
+``--workload sweep`` prints a table of further sizes (decode over batch sizes and contexts up to
+8,192 tokens, prompts of 64 to 8,192 tokens whole and in chunks of 256) instead of the JSON line.
 """
 
 import argparse
@@ -379,6 +381,70 @@ def run_generation(args):
     }
 
 
+def run_sweep(args):
+    """Further sizes: decode steps over batch sizes and context lengths, prompts of many lengths
+    whole and in chunks of 256.  GPT-2 XL's layer sizes with room for 8,192 positions and
+    ``--layers`` layers (12 unless given: the cache of 64 sequences of 8,192 tokens through 48 layers
+    would be 160 GB); every line is tab-separated text, not the one JSON line of the default run."""
+    import torch
+
+    import burn_transformers_amd as bt
+    layers = args.layers if args.layers != XL["n_layer"] else 12
+    dtype = args.dtype or "bf16"
+    config = dict(XL, n_layer=layers, n_positions=8192)
+    model = build_model(config, dtype)
+    vocab = config["vocab_size"]
+    weight_bytes, kv_per_token, _ = model_bytes_and_flops(config, layers, dtype)
+    d, m = config["n_embd"], config["n_inner"]
+    per_layer = 3 * d * d + d * d + 2 * d * m
+    print(f"# GPT-2 XL layer sizes, {layers} layers, 8,192 positions, {dtype}, random weights")
+    print("# decode: one token per sequence from a HIP graph, every sequence holding `context` tokens")
+    print("kind\tbatch\tcontext\tms_per_step\ttokens_per_s\thbm_fraction")
+    for context in (1024, 2048, 4096, 8192):
+        for batch in (1, 8, 16, 32, 64):
+            engine = bt.Engine(model, max_tokens=batch * (context + 64))
+            slots = [engine.open() for _ in range(batch)]
+            prompts = synthetic_prompts(batch, context - 23, vocab, seed=context + batch)
+            for begin in range(0, batch, 4):
+                engine.step([(slots[i], prompts[i]) for i in range(begin, min(begin + 4, batch))], want=[[] for _ in range(begin, min(begin + 4, batch))])
+            ids = [7] * batch
+            for _ in range(8):
+                engine.step([(slot, [token]) for slot, token in zip(slots, ids)])
+            groups = []
+            for _ in range(3):                       # the median of three groups of five steps
+                torch.cuda.synchronize()
+                started = time.perf_counter()
+                for _ in range(5):
+                    engine.step([(slot, [token]) for slot, token in zip(slots, ids)])
+                torch.cuda.synchronize()
+                groups.append((time.perf_counter() - started) / 5)
+            seconds = sorted(groups)[1]
+            nbytes = weight_bytes + batch * context * kv_per_token
+            print(f"decode\t{batch}\t{context}\t{seconds * 1e3:.3f}\t{batch / seconds:.0f}\t{nbytes / seconds / 1e9 / PEAK_HBM_GBS:.3f}", flush=True)
+            del engine
+    print("# prompts: one sequence, whole (chunk 0) or in chunks; the fraction is of the MFMA peak")
+    print("kind\ttokens\tchunk\tms\ttokens_per_s\tmfma_fraction")
+    engine = bt.Engine(model, max_tokens=8192 + 64)
+    for tokens in (64, 128, 256, 512, 1024, 2048, 4096, 8192):
+        for chunk in (0, 256):
+            if chunk and tokens <= chunk:
+                continue
+            prompt = synthetic_prompts(1, tokens, vocab, seed=tokens)[0]
+            times = []
+            for _ in range(5):
+                slot = engine.open()
+                torch.cuda.synchronize()
+                started = time.perf_counter()
+                for begin in range(0, tokens, chunk or tokens):
+                    engine.step([(slot, prompt[begin:begin + (chunk or tokens)])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - started)
+                engine.close(slot)
+            seconds = sorted(times)[1]
+            flops = 2.0 * tokens * layers * per_layer + layers * 2.0 * d * tokens * (tokens + 1) + 2.0 * d * vocab
+            print(f"prompt\t{tokens}\t{chunk}\t{seconds * 1e3:.3f}\t{tokens / seconds:.0f}\t{flops / seconds / PEAK_FLOPS[dtype]:.3f}", flush=True)
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -388,7 +454,7 @@ def main():
     parser.add_argument("--layers", type=int, default=XL["n_layer"], help="fewer layers than the 48 of GPT-2 XL")
     parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
     parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
-    parser.add_argument("--workload", choices=["xl", "small", "medium"], default="xl")
+    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep"], default="xl")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     parser.add_argument("--no-kernels", action="store_true", help="skip the classes of kernels on their own")
     args = parser.parse_args()
@@ -397,7 +463,9 @@ def main():
         sys.exit(2)
     if args.repetitions < 1:
         parser.error("--repetitions must be at least 1")
-    if args.workload == "xl":
+    if args.workload == "sweep":
+        run_sweep(args)
+    elif args.workload == "xl":
         args.dtype = args.dtype or "bf16"
         print(json.dumps(run_xl(args)))
     else:

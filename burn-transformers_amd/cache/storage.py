@@ -5,8 +5,9 @@ Cache entries (one per layer that keeps keys and values, as the model's schedule
 with the same :class:`KVSpec` form a *group* with storage of its own:
     [entries, blocks, kv_heads, 2, 64 * head_dim]: for each block and head the plane of its keys,
     [64, head_dim], beside the plane of its values, [16, head_dim, 4] (four positions interleaved)
-All groups share one block table per sequence, because a sequence is equally long in all of
-them.  Fixed-size state ([entries, slots, *shape], zeroed when a slot is handed out) lives beside
+Every group has block lists and a block table of its own: a sequence is equally long in all of
+them, but a group that reads only a window of the latest positions gives the blocks behind the
+window back while the sequence is still growing.  Fixed-size state ([entries, slots, *shape], zeroed when a slot is handed out) lives beside
 it for mixers that carry state instead of, or in addition to, keys and values.
 """
 
@@ -103,8 +104,8 @@ class Cache:
             for index, entry in enumerate(entries):
                 self.state_entry[entry] = (len(self.state_groups), index)
             self.state_groups.append(group)
-        # one block table serves every group: the ledger runs a single list of block numbers
-        self.ledger = CacheLedger(1 if self.kv_groups else 0, n_blocks, self.max_slots, self.max_blocks)
+        self.ledger = CacheLedger(len(self.kv_groups), n_blocks, self.max_slots, self.max_blocks,
+                                  windows=[group.spec.window for group in self.kv_groups])
 
     # --- slots -----------------------------------------------------------------------------
     def acquire(self):
@@ -126,13 +127,23 @@ class Cache:
     def length(self, slot):
         return self.ledger.lengths[slot]
 
-    def blocks(self, slot):
-        return self.ledger.held_blocks[0][slot] if self.kv_groups else []
+    def blocks(self, slot, group=0):
+        """The blocks a sequence holds in one group, by block number (RELEASED where a window has
+        moved on)."""
+        return self.ledger.held_blocks[group][slot] if self.kv_groups else []
+
+    def block_rows(self, slots):
+        """For a step's block tables: [group][sequence] -> block list, a released block's place
+        filled with block 0 (a valid block that no kernel reads for this sequence: a query's keys
+        start inside its window)."""
+        return [[[block if block >= 0 else 0 for block in self.ledger.held_blocks[group][slot]] for slot in slots]
+                for group in range(len(self.kv_groups))]
 
     # --- views -----------------------------------------------------------------------------
-    def kv_view(self, entry, block_table):
+    def kv_view(self, entry, block_tables):
+        """``block_tables``: the step's tables [groups, n_seqs, max_blocks]."""
         group, index = self.kv_entry[entry]
-        return self.kv_groups[group].view(index, block_table, self.max_blocks)
+        return self.kv_groups[group].view(index, block_tables[group], self.max_blocks)
 
     def state(self, entry):
         """[slots, *shape] state of a cache entry."""

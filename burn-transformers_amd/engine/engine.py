@@ -153,8 +153,7 @@ class Engine:
             ledger.reserve(slot, length)
         try:
             plan = StepPlan(checked["slots"], checked["starts"], checked["counts"], checked["ids"],
-                            checked["wanted"], [self.cache.blocks(s) for s in checked["slots"]],
-                            self.cache.max_blocks)
+                            checked["wanted"], self.cache.block_rows(checked["slots"]), self.cache.max_blocks)
             if self.use_graphs:
                 logits = self._run_from_graph(plan, readout=bool(checked["wanted"]))
             else:

@@ -5,7 +5,9 @@ A step is a set of sequences, each bringing ``count`` new tokens that start at p
 sequence and position.  All integer tables of a step travel to the GPU in ONE copy, as
 sections of one int32 buffer:
 
-    tok_ids[T] tok_pos[T] tok_seq[T] seq_off[B+1] seq_start[B] slots[B] sel_rows[R] block_table[B*max_blocks]
+    tok_ids[T] tok_pos[T] tok_seq[T] seq_off[B+1] seq_start[B] slots[B] sel_rows[R] block_table[G*B*max_blocks]
+
+(G: the groups of layers of the cache, each with a block table of its own.)
 """
 
 import numpy as np
@@ -21,30 +23,33 @@ def _align(n):
 class StepLayout:
     """Offsets of the sections for T tokens, B sequences, R wanted rows."""
 
-    def __init__(self, tokens, seqs, rows, max_blocks):
-        self.tokens, self.seqs, self.rows, self.max_blocks = tokens, seqs, rows, max_blocks
+    def __init__(self, tokens, seqs, rows, max_blocks, groups=1):
+        self.tokens, self.seqs, self.rows, self.max_blocks, self.groups = tokens, seqs, rows, max_blocks, groups
         offset = 0
         self.sections = {}
         for name, size in (("tok_ids", tokens), ("tok_pos", tokens), ("tok_seq", tokens),
                            ("seq_off", seqs + 1), ("seq_start", seqs), ("slots", seqs),
-                           ("sel_rows", rows), ("block_table", seqs * max_blocks)):
+                           ("sel_rows", rows), ("block_table", groups * seqs * max_blocks)):
             self.sections[name] = (offset, size)
             offset = _align(offset + size)
         self.total = offset
 
     def key(self):
-        return (self.tokens, self.seqs, self.rows, self.max_blocks)
+        return (self.tokens, self.seqs, self.rows, self.max_blocks, self.groups)
 
 
 class StepPlan:
     """A validated step on the host: nothing on the GPU or in the cache has changed yet."""
 
     def __init__(self, slots, starts, counts, token_ids, wanted, block_rows, max_blocks):
+        """``block_rows[group][sequence]``: the blocks of each of the step's sequences in each group
+        of the cache (``Cache.block_rows``)."""
         self.slots, self.starts, self.counts = slots, starts, counts
         self.n_seqs, self.n_tokens = len(slots), int(sum(counts))
         self.max_count = int(max(counts))
         self.decode = self.max_count == 1
-        self.layout = StepLayout(self.n_tokens, self.n_seqs, len(wanted), max_blocks)
+        groups = max(len(block_rows), 1)
+        self.layout = StepLayout(self.n_tokens, self.n_seqs, len(wanted), max_blocks, groups)
         host = np.zeros(self.layout.total, dtype=np.int32)
         section = lambda name: host[self.layout.sections[name][0]:sum(self.layout.sections[name])]
         section("tok_ids")[:] = token_ids
@@ -59,9 +64,10 @@ class StepPlan:
         section("seq_start")[:] = starts
         section("slots")[:] = slots
         section("sel_rows")[:] = wanted
-        table = section("block_table").reshape(self.n_seqs, max_blocks)
-        for row, blocks in enumerate(block_rows):
-            table[row, :len(blocks)] = blocks
+        table = section("block_table").reshape(groups, self.n_seqs, max_blocks)
+        for group, rows in enumerate(block_rows):
+            for row, blocks in enumerate(rows):
+                table[group, row, :len(blocks)] = blocks
         self.host = host
         self.new_lengths = {slot: start + count for slot, start, count in zip(slots, starts, counts)}
         self.context_limit = min(context_limit(max(self.new_lengths.values())), max_blocks * BLOCK)
@@ -91,7 +97,8 @@ class Step:
         self.n_tokens, self.n_seqs, self.max_blocks = layout.tokens, layout.seqs, layout.max_blocks
         for name, (offset, size) in layout.sections.items():
             setattr(self, name, device_meta[offset:offset + size])
-        self.block_table = self.block_table.view(self.n_seqs, self.max_blocks) if self.n_seqs else self.block_table
+        if self.n_seqs:       # [groups, sequences, blocks]; a mixer gets its group's table with its view of the cache
+            self.block_table = self.block_table.view(layout.groups, self.n_seqs, self.max_blocks)
         self.dtype = dtype
         self.dtype_is_bf16 = dtype == torch.bfloat16
         self.pool = pool

@@ -15,9 +15,9 @@ def make_step(dtype, counts, starts=None, ids=None, wanted=None, cache=None, slo
     ids = np.asarray(ids if ids is not None else np.zeros(total), dtype=np.int64)
     wanted = list(wanted) if wanted is not None else [int(x) - 1 for x in np.cumsum(counts)]
     if cache is not None:
-        rows, max_blocks = [cache.blocks(s) for s in slots], cache.max_blocks
+        rows, max_blocks = cache.block_rows(slots), cache.max_blocks
     else:
-        rows, max_blocks = [[] for _ in slots], 1
+        rows, max_blocks = [[[] for _ in slots]], 1
     plan = StepPlan(slots, starts, list(counts), ids, wanted, rows, max_blocks)
     meta = torch.from_numpy(plan.host).to(device)
     return Step(plan.layout, meta, pool or BufferPool(torch.device(device)), dtype, plan)

@@ -118,3 +118,79 @@ def test_truncate_gives_blocks_back_and_keeps_the_rest():
     ledger.reserve(a, 130)
     ledger.commit(a, 130)
     ledger.check()
+
+
+def test_a_group_with_a_window_gives_blocks_back_while_the_sequence_grows():
+    """Two groups: one keeps every key, one reads only the last 100 positions.  The second gives a
+    block back as soon as the next token can no longer read any of its positions; the first keeps
+    all; both have free lists of their own."""
+    from burn_transformers_amd.cache.ledger import RELEASED
+    ledger = CacheLedger(2, blocks_per_group=8, max_slots=2, max_blocks_per_sequence=8, windows=[0, 100])
+    a = ledger.acquire()
+    length = 0
+    for grow in (60, 70, 40, 1, 1, 90, 150, 30):
+        length += grow
+        ledger.check_growth({a: length})
+        ledger.reserve(a, length)
+        ledger.commit(a, length)
+        ledger.check()
+        blocks = (length + BLOCK - 1) // BLOCK
+        first = max(0, length - 100 + 1) // BLOCK           # the block of the oldest position the next token reads
+        full, windowed = ledger.held_blocks[0][a], ledger.held_blocks[1][a]
+        assert len(full) == blocks and RELEASED not in full
+        assert windowed[:first] == [RELEASED] * first and RELEASED not in windowed[first:] and len(windowed) == blocks
+        assert ledger.blocks[0].available() == 8 - blocks and ledger.blocks[1].available() == 8 - (blocks - first)
+    assert length == 442 and ledger.blocks[1].available() == 6      # 7 blocks long, 2 of them still held
+    # a second sequence can use what the window gave back, though the first group is nearly full
+    b = ledger.acquire()
+    with pytest.raises(CacheFull, match="needs 2 more blocks"):
+        ledger.check_growth({b: 100})                      # the group that keeps everything has one block left
+    ledger.check_growth({b: 64})
+    ledger.reserve(b, 64)
+    ledger.commit(b, 64)
+    ledger.check()
+    # rewinding: fine while the shorter sequence reads nothing that is gone, refused otherwise, and
+    # a refusal changes nothing
+    before = ([list(x) for x in ledger.held_blocks[0]], [list(x) for x in ledger.held_blocks[1]], list(ledger.lengths))
+    with pytest.raises(ValueError, match="window of 100 has given the blocks before it back"):
+        ledger.truncate(a, 300)
+    assert ([list(x) for x in ledger.held_blocks[0]], [list(x) for x in ledger.held_blocks[1]], list(ledger.lengths)) == before
+    ledger.truncate(a, 420)                                 # reads back to 321: block 5, which is still there
+    assert ledger.lengths[a] == 420 and len(ledger.held_blocks[1][a]) == 7
+    ledger.check()
+    ledger.release(a)
+    ledger.release(b)
+    ledger.check()
+    assert [f.available() for f in ledger.blocks] == [8, 8]
+
+
+def test_random_traffic_with_windows_keeps_the_books():
+    rng = random.Random(7)
+    ledger = CacheLedger(3, blocks_per_group=30, max_slots=6, max_blocks_per_sequence=10, windows=[0, 64, 200])
+    live = {}
+    for _ in range(600):
+        action = rng.random()
+        if action < 0.2 and ledger.slots.available():
+            live[ledger.acquire()] = 0
+        elif action < 0.3 and live:
+            slot = rng.choice(list(live))
+            ledger.release(slot)
+            del live[slot]
+        elif live:
+            slot = rng.choice(list(live))
+            target = min(live[slot] + rng.randint(1, 150), 640)
+            try:
+                ledger.check_growth({slot: target})
+            except CacheFull:
+                continue
+            ledger.reserve(slot, target)
+            if rng.random() < 0.1:                          # a pass that failed: the reservation is undone
+                ledger.truncate(slot, live[slot])
+            else:
+                ledger.commit(slot, target)
+                live[slot] = target
+        ledger.check()
+    for slot in list(live):
+        ledger.release(slot)
+    ledger.check()
+    assert all(f.available() == 30 for f in ledger.blocks)

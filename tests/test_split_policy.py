@@ -68,7 +68,7 @@ def test_decode_runs_at_measured_sizes(monkeypatch):
 def test_context_classes():
     from burn_transformers_amd.engine.step import StepPlan, context_limit
     assert [context_limit(n) for n in (1, 1024, 1025, 2048, 2049, 5000)] == [1024, 1024, 2048, 2048, 4096, 8192]
-    plan = StepPlan([0, 1], [10, 3000], [1, 1], [5, 6], [0, 1], [[0], list(range(47))], 128)
+    plan = StepPlan([0, 1], [10, 3000], [1, 1], [5, 6], [0, 1], [[[0], list(range(47))]], 128)
     assert plan.context_limit == 4096 and plan.decode
     # never more than a sequence can hold (3 blocks of 64 tokens here)
-    assert StepPlan([0], [100], [1], [5], [0], [[0, 1]], 3).context_limit == 192
+    assert StepPlan([0], [100], [1], [5], [0], [[[0, 1]]], 3).context_limit == 192

@@ -189,15 +189,15 @@ def kernel_classes(engine, entries, attention_bytes, attention_flops, peak_flops
     from burn_transformers_amd.kernels import library as K
     if not engine.use_programs:
         return {}
-    before = set(engine._programs)
     graphs, engine.use_graphs = engine.use_graphs, False
     try:
         engine.step(entries)
         torch.cuda.synchronize()
     finally:
         engine.use_graphs = graphs
-    fresh = [key for key in engine._programs if key not in before] or list(engine._programs)[-1:]
-    program = engine._programs[fresh[-1]][0]
+    program = engine.last_program
+    if program is None:          # the step made a workspace grow, and a list recorded meanwhile is not kept
+        return {}
     classes = {}
     for lib, name, call in program.calls:
         label, nbytes, flops = _class_of(name, call)

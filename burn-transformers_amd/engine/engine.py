@@ -55,6 +55,7 @@ class Engine:
         self._programs = {}                # shape -> (Program, logits), in order of last use
         self._programs_generation = -1     # the workspace generation the lists were recorded for
         self.program_runs = 0
+        self.last_program = None           # the launch list of the latest step, if it ran from one or left one
         self._meta = None                  # device int32 buffer of eager steps
         self._pinned = []                  # ring of (pinned int32 tensor, event)
         self._pinned_next = 0
@@ -202,9 +203,10 @@ class Engine:
         return self.model.forward(step, self.cache)
 
     def _run_program(self, plan, readout):
-        """The step from its launch list: recorded the first time a shape comes (the parts run as
-        always, but every kernel call is kept instead of launched), walked in C++ every time.  A
-        list names workspaces by address, so a workspace that had to grow makes all lists stale."""
+        """The step from its launch list.  The first time a shape comes the parts run as always and
+        launch as they go (the GPU starts at once), and every kernel call is kept as well; from
+        then on the list is walked in C++.  A list names workspaces by address, so a workspace that
+        had to grow makes all lists stale, and a list recorded while one grew is not kept."""
         if self._programs_generation != self.pool.generation:
             self._programs.clear()
             self._programs_generation = self.pool.generation
@@ -212,26 +214,28 @@ class Engine:
         held = self._programs.pop(key, None)
         if held is None:
             step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
-            for _ in range(4):
-                # a workspace that grows WHILE the list is recorded leaves its old address in the calls
-                # recorded before: record again, now that it is large enough from the start
-                generation = self.pool.generation
-                program = K.Program()
-                with program.recording():
-                    logits = self.model.forward(step, self.cache, readout=readout)
-                if self.pool.generation == generation:
-                    break
-            else:
-                raise RuntimeError("the workspaces of a step did not settle while its launch list was recorded")
+            generation = self.pool.generation
+            program = K.Program()
+            with program.recording(launch=True):
+                logits = self.model.forward(step, self.cache, readout=readout)
             if not readout:
                 logits = torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
-            if self._programs_generation != self.pool.generation:      # recording made a workspace grow:
-                self._programs.clear()                                 # the lists before this one are stale
+            self.last_program = None
+            if self.pool.generation != generation:
+                # A workspace grew while the step ran.  The launches themselves were in order and are
+                # right, but calls recorded before the growth name the old address, and so do all
+                # older lists: none is kept, and the shape records again when it next comes (the
+                # workspaces are then large enough from the start).
+                self._programs.clear()
                 self._programs_generation = self.pool.generation
-            held = (program, logits)
+                return logits
             while len(self._programs) >= _MAX_PROGRAMS:
                 self._programs.pop(next(iter(self._programs)))
+            self._programs[key] = (program, logits)
+            self.last_program = program
+            return logits
         self._programs[key] = held                        # (again) the most recently used
+        self.last_program = held[0]
         held[0].run()
         self.program_runs += 1
         return held[1]

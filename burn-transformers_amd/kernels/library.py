@@ -195,7 +195,8 @@ def _launch(lib, name, call):
     program = _recorder[0]
     if program is not None:
         program.add(lib, name, call)
-        return
+        if not program.launch_while_recording:
+            return
     _check(lib, getattr(lib, name)(_stream(), ctypes.byref(call)))
 
 
@@ -209,6 +210,9 @@ class Program:
             model.forward(step, cache)        # nothing is launched; every kernels.library call is kept
         program.run()                         # launches them all, now and as often as wanted
 
+    ``recording(launch=True)`` keeps the calls AND launches each as it comes: the first step of a
+    shape then starts on the GPU at once, as it would without a list, and leaves its list behind.
+
     What the list holds is only addresses and sizes: it stays valid as long as every buffer, table
     and weight it names stays where it is, and gives the same results as calling the kernels one
     by one, bit for bit (they are the same calls)."""
@@ -216,12 +220,14 @@ class Program:
     def __init__(self):
         self.calls = []             # (module, entry point name, structure); the structures are kept alive here
         self._entries = None
+        self.launch_while_recording = False
 
     def add(self, lib, name, call):
         self.calls.append((lib, name, call))
         self._entries = None
 
-    def recording(self):
+    def recording(self, launch=False):
+        self.launch_while_recording = launch
         return _Recording(self)
 
     def __len__(self):

@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 MAX_HEADER_BYTES = 100 * 10 ** 6     # src/checkpoint/options.rs:69-81
+MAX_TENSORS = 10 * 10 ** 6
 MAX_RANK = 32
 
 DTYPES = {
@@ -57,6 +58,8 @@ def read_header(path):
             raise SafetensorsError(f"{path}: header is not JSON ({error})") from error
     if not isinstance(header, dict):
         raise SafetensorsError(f"{path}: header must be an object")
+    if len(header) > MAX_TENSORS:
+        raise SafetensorsError(f"{path}: {len(header)} tensors, at most {MAX_TENSORS} are read")
     payload_start = 8 + header_len
     payload_size = size - payload_start
     entries, ranges = {}, []
@@ -77,10 +80,16 @@ def read_header(path):
                 f"{path}: tensor {name!r} {dtype}{list(shape)} needs {want} bytes, its range is [{begin}, {end})")
         entries[name] = Entry(name, dtype, shape, begin, end, path, payload_start)
         ranges.append((begin, end, name))
+    # the ranges tile the payload: they start at its first byte, follow each other without overlap
+    # or gap, and end at its last (src/checkpoint/artifact.rs:1-11)
     ranges.sort()
     for (_, end_a, name_a), (begin_b, _, name_b) in zip(ranges, ranges[1:]):
         if begin_b < end_a:
             raise SafetensorsError(f"{path}: tensors {name_a!r} and {name_b!r} overlap")
+        if begin_b > end_a:
+            raise SafetensorsError(f"{path}: {begin_b - end_a} bytes between tensors {name_a!r} and {name_b!r} belong to no tensor")
+    if ranges and (ranges[0][0] != 0 or ranges[-1][1] != payload_size):
+        raise SafetensorsError(f"{path}: the tensors cover bytes [{ranges[0][0]}, {ranges[-1][1]}) of a payload of {payload_size}")
     return entries
 
 

@@ -54,6 +54,16 @@ def test_malformed_files_are_refused_before_any_payload(tmp_path):
         f.write(struct.pack("<Q", len(header)) + header + b"\0" * 12)
     with pytest.raises(SafetensorsError, match="overlap"):
         read_header(path)
+    # the ranges must tile the payload: no gap between tensors, none before the first, none after the last
+    for offsets, size, message in (([[0, 8], [12, 20]], 20, "4 bytes between tensors 'a' and 'b' belong to no tensor"),
+                                   ([[4, 12], [12, 20]], 20, r"cover bytes \[4, 20\) of a payload of 20"),
+                                   ([[0, 8], [8, 16]], 24, r"cover bytes \[0, 16\) of a payload of 24")):
+        header = json.dumps({"a": {"dtype": "F32", "shape": [2], "data_offsets": offsets[0]},
+                             "b": {"dtype": "F32", "shape": [2], "data_offsets": offsets[1]}}).encode()
+        with open(path, "wb") as f:
+            f.write(struct.pack("<Q", len(header)) + header + b"\0" * size)
+        with pytest.raises(SafetensorsError, match=message):
+            read_header(path)
     with open(path, "wb") as f:
         f.write(struct.pack("<Q", 10 ** 12))
     with pytest.raises(SafetensorsError, match="does not fit"):

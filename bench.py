@@ -5,8 +5,9 @@
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
 sequences, prefilled with 512 synthetic tokens each, is decoded towards 1,024.  A step is one
-decode step of the whole batch: the engine's step function followed by greedy selection and the
-readback of the chosen ids, exactly what the generation loop runs.  With no flags, 16 untimed and
+decode step of the whole batch: the engine's step function, greedy selection and the readback of
+the chosen ids, exactly what the generation loop runs (the ids feed the next step from the GPU,
+and the host reads them while that step runs).  With no flags, 16 untimed and
 495 timed steps take the sequences from 512 to 1,024 tokens.
 
 The protocol is the reference's (BENCHMARKS.md:71-87, tests/support/causal_decode_benchmark.rs:
@@ -95,21 +96,26 @@ def decode_repetition(engine, batch, warmup, steps, vocab, seed):
     for begin in range(0, batch, 8):
         part = engine.step([(slots[i], prompts[i]) for i in range(begin, min(begin + 8, batch))])
         logits[begin:begin + part.shape[0]] = part
-    ids, _ = sampler.select(logits, rows)
+    sampler.launch(logits, rows)
+    entries = [(slot, [0]) for slot in slots]
 
-    def one_step(ids):
-        logits = engine.step([(slot, [token]) for slot, token in zip(slots, ids)])
-        return sampler.select(logits, rows)[0]
+    def one_step():
+        # as the generation loop decodes: the chosen ids feed the step from the GPU, and the host
+        # reads them (the step's one readback) while the step runs
+        logits = engine.step(entries, device_tokens=sampler.device_ids(batch))
+        sampler.result()
+        sampler.launch(logits, rows)
 
     for _ in range(warmup):
-        ids = one_step(ids)
+        one_step()
     first_context = engine.length(slots[0])
     torch.cuda.synchronize()
     started = time.perf_counter()
     for _ in range(steps):
-        ids = one_step(ids)
+        one_step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
+    sampler.result()
     for slot in slots:
         engine.close(slot)
     return elapsed, first_context

@@ -144,17 +144,28 @@ class Engine:
         # block rows are read after the reservation, in `step`
         return dict(slots=slots, starts=starts, counts=counts, ids=ids, wanted=wanted, new_lengths=new_lengths)
 
-    def step(self, entries, want=None):
+    def step(self, entries, want=None, device_tokens=None):
         """Runs one step; returns float32 logits [wanted places, vocab] on the GPU, valid until the
         next step.  ``entries``: [(slot, token ids)], ``want``: per entry the places among its
-        tokens whose logits are wanted (default: each entry's last token)."""
+        tokens whose logits are wanted (default: each entry's last token).
+
+        ``device_tokens``: for a step of one token per sequence, an int32 tensor on the GPU that
+        holds the tokens themselves, in the order of the entries (whose own token is then only a
+        placeholder): what a selection kernel has just chosen can feed the next step before the
+        host has read it, so the host's work on a step overlaps the GPU's work on the one before.
+        The ids are not validated (a selection cannot choose outside the vocabulary)."""
         checked = self.plan(entries, want)
+        if device_tokens is not None:
+            if max(checked["counts"]) != 1 or device_tokens.numel() != len(entries) or \
+                    device_tokens.dtype != torch.int32 or device_tokens.device != self.device:
+                raise StepError("device_tokens: one int32 token on this GPU for each sequence of a step of single tokens")
         ledger = self.cache.ledger
         for slot, length in checked["new_lengths"].items():
             ledger.reserve(slot, length)
         try:
             plan = StepPlan(checked["slots"], checked["starts"], checked["counts"], checked["ids"],
                             checked["wanted"], self.cache.block_rows(checked["slots"]), self.cache.max_blocks)
+            plan.device_tokens = device_tokens
             if self.use_graphs:
                 logits = self._run_from_graph(plan, readout=bool(checked["wanted"]))
             else:
@@ -189,11 +200,18 @@ class Engine:
         device_meta[:host.size].copy_(entry[0][:host.size], non_blocking=True)
         entry[1].record()
 
+    def _upload_plan(self, plan, device_meta):
+        """The step's tables, and over their token ids the tokens that are on the GPU already."""
+        self._upload(plan.host, device_meta)
+        if plan.device_tokens is not None:
+            offset, size = plan.layout.sections["tok_ids"]
+            device_meta[offset:offset + size].copy_(plan.device_tokens, non_blocking=True)
+
     def _run_eager(self, plan, want_logits=True):
         if self._meta is None or self._meta.numel() < plan.layout.total:
             self._meta = torch.empty(max(plan.layout.total * 2, _META_WORDS), dtype=torch.int32, device=self.device)
             self._programs.clear()                        # they name the old tables
-        self._upload(plan.host, self._meta)
+        self._upload_plan(plan, self._meta)
         if self.use_programs:
             return self._run_program(plan, want_logits)
         step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
@@ -258,7 +276,7 @@ class Engine:
             while len(self._graphs) >= _MAX_GRAPHS:
                 self._graphs.pop(next(iter(self._graphs)))
         self._graphs[key] = held                          # (again) the most recently used
-        self._upload(plan.host, held["meta"])
+        self._upload_plan(plan, held["meta"])
         held["graph"].replay()
         self.graph_replays += 1
         return held["logits"]

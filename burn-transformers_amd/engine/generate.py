@@ -91,6 +91,9 @@ def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None, l
             if final:
                 logits.index_copy_(0, torch.tensor(final, device=engine.device), chunk_logits)
         live = list(range(len(prompts)))
+        if sampler.pipelined:
+            _decode_ahead(engine, sampler, tracker, slots, open_rows, logits, live, on_token)
+            return tracker.sequences
         while True:
             ids, logps = sampler.select(logits, live)
             next_live, next_entries = [], []
@@ -114,6 +117,50 @@ def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None, l
         for row in open_rows:
             engine.close(slots[row])
     return tracker.sequences
+
+
+def _decode_ahead(engine, sampler, tracker, slots, open_rows, logits, live, on_token):
+    """The decode loop with the host one step behind the GPU.  A selection's ids stay on the GPU and
+    feed the next step from there (``Engine.step(device_tokens=...)``); the host reads them while
+    that step runs, so its own work (stop rules, the next step's tables) costs the GPU no idle
+    time.  A row whose token turns out to end it (end-of-sequence, a stop sequence) has then been
+    fed once too often: that position goes with the row's slot.  Rows that end by their length are
+    known beforehand and are not fed.  Tokens, log-probabilities and finish reasons are those of
+    the loop that waits for every token (the same kernels on the same rows; a row's logits do not
+    depend on what else is in the batch beyond rounding)."""
+    device = engine.device
+    while True:
+        sampler.launch(logits, live)
+        # rows that go on unless this very token stops them
+        ahead = [row for row in live if len(tracker.sequences[row].token_ids) + 1 < tracker.limit(row)]
+        next_logits = None
+        if ahead:
+            tokens = sampler.device_ids(len(live))
+            if len(ahead) != len(live):
+                going = set(ahead)
+                places = [i for i, row in enumerate(live) if row in going]
+                tokens = tokens[torch.tensor(places, device=device)]
+            next_logits = engine.step([(slots[row], [0]) for row in ahead], device_tokens=tokens)
+        ids, logps = sampler.result()
+        next_live = []
+        for row, token, logp in zip(live, ids, logps):
+            if not math.isfinite(logp):
+                raise GenerationError(f"row {row}: the selected token has a non-finite log-probability")
+            reason = tracker.push(row, token, logp)
+            if on_token is not None:
+                on_token(row, token, logp, reason)
+            if reason is None:
+                next_live.append(row)
+            else:                                   # the sequence leaves the batch; its slot is free again
+                engine.close(slots[row])
+                open_rows.discard(row)
+        if not next_live:
+            return
+        if len(next_live) != len(ahead):            # a token ended its row: that row's logits are dropped
+            kept = set(next_live)
+            places = [i for i, row in enumerate(ahead) if row in kept]
+            next_logits = next_logits[torch.tensor(places, device=device)]
+        logits, live = next_logits, next_live
 
 
 def generate(engine, prompts, config=None, prefill_chunk=None, batch_size=None, on_token=None, total_length=None):

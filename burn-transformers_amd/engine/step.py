@@ -69,6 +69,7 @@ class StepPlan:
             for row, blocks in enumerate(rows):
                 table[group, row, :len(blocks)] = blocks
         self.host = host
+        self.device_tokens = None      # set by the engine: the tokens, where they are on the GPU already
         self.new_lengths = {slot: start + count for slot, start, count in zip(slots, starts, counts)}
         self.context_limit = min(context_limit(max(self.new_lengths.values())), max_blocks * BLOCK)
 

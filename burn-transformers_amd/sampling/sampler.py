@@ -40,6 +40,8 @@ class Sampler:
         self.packed = torch.zeros((2, batch_rows), dtype=torch.int32, device=device)
         self.ids, self.logp = self.packed[0], self.packed[1].view(torch.float32)
         self.host = torch.zeros((2, batch_rows), dtype=torch.int32).pin_memory()
+        self._arrived = torch.cuda.Event()     # the copy of the latest selection into `host`
+        self._launched = 0                     # rows of the selection that `result` has not fetched yet
         self.history = self.bias = None
         if vocabulary_size is not None and config.processes_logits(vocabulary_size):
             from .history import TokenHistory
@@ -51,20 +53,50 @@ class Sampler:
                     bias[token] = value
                 self.bias = bias.to(device)
 
+    @property
+    def pipelined(self):
+        """True where a selection needs nothing from the host but the rows' numbers: it can then be
+        started (``launch``) and fetched later (``result``), and the chosen ids can feed the next
+        step from the GPU (``device_ids``) before the host has seen them."""
+        return self.history is None
+
+    def launch(self, logits, rows):
+        """Starts the selection of one token per row and its copy to the host; returns at once."""
+        if self.history is not None:
+            raise RuntimeError("a selection that depends on what the rows have held so far cannot run ahead of the host")
+        count = len(rows)
+        config = self.config
+        draw_rows = None
+        if config.sampling:
+            draw_rows = torch.tensor(rows, dtype=torch.int32).to(self.device, non_blocking=True)
+        K.sample(logits, self.ids[:count], self.logp[:count],
+                 temperature=float(config.temperature) if config.sampling else None,
+                 seed=config.seed, first_draw=self.selections * self.batch_rows, draw_rows=draw_rows)
+        self.selections += 1
+        self.host.copy_(self.packed, non_blocking=True)
+        self._arrived.record()
+        self._launched = count
+
+    def device_ids(self, count):
+        """The ids of the latest selection where they were chosen: int32 [count] on the GPU."""
+        return self.ids[:count]
+
+    def result(self):
+        """(ids, log-probabilities) of the selection ``launch`` started, as Python lists; waits for
+        their copy.  This is the step's one readback."""
+        count, self._launched = self._launched, 0
+        self._arrived.synchronize()
+        return self.host[0, :count].tolist(), self.host[1].view(torch.float32)[:count].tolist()
+
     def select(self, logits, rows):
         """One token for each row of ``logits`` (float32 [len(rows), vocab]); ``rows`` are the rows'
-        numbers in the batch as it started.  Returns (ids, log-probabilities) as Python lists; this
-        is the step's one readback."""
+        numbers in the batch as it started.  Returns (ids, log-probabilities) as Python lists."""
         count = len(rows)
         config = self.config
         first_draw = self.selections * self.batch_rows
         if self.history is None:
-            draw_rows = None
-            if config.sampling:
-                draw_rows = torch.tensor(rows, dtype=torch.int32).to(self.device, non_blocking=True)
-            K.sample(logits, self.ids[:count], self.logp[:count],
-                     temperature=float(config.temperature) if config.sampling else None,
-                     seed=config.seed, first_draw=first_draw, draw_rows=draw_rows)
+            self.launch(logits, rows)
+            return self.result()
         else:
             # one small upload: the rows' numbers, then where each row's banned tokens start, then those
             banned = [self.history.banned(row) for row in rows]

@@ -73,6 +73,11 @@ class GenerationTracker:
         sequence.finish_reason = stop_decision(self.config, sequence.token_ids, self.limits[row])
         return sequence.finish_reason
 
+    def limit(self, row):
+        """The most new tokens the row may get."""
+        own = self.limits[row]
+        return self.config.max_new_tokens if own is None else min(own, self.config.max_new_tokens)
+
     def finished(self, row):
         return self.sequences[row].finish_reason is not None
 

@@ -446,6 +446,37 @@ def test_refused_steps_change_nothing():
 
 
 @pytest.mark.parametrize("graphs", [False, True])
+def test_tokens_that_are_on_the_gpu_already_feed_a_step_from_there(graphs):
+    """``device_tokens``: the step reads its tokens from a tensor on the GPU (what a selection has
+    just chosen) instead of from the entries; same logits, bit for bit, as the same tokens given
+    by the host, also when the step is replayed from a graph."""
+    from burn_transformers_amd.engine.engine import StepError
+    name = "A"
+    by_host, by_device = engine_for(name, "bfloat16", graphs=graphs), engine_for(name, "bfloat16", graphs=graphs)
+    requests = prompts_for(name, [30, 9, 50], seed=90)
+    slots_h = [by_host.open() for _ in requests]
+    slots_d = [by_device.open() for _ in requests]
+    by_host.step([(s, r[:5]) for s, r in zip(slots_h, requests)])
+    by_device.step([(s, r[:5]) for s, r in zip(slots_d, requests)])
+    for t in range(5, 9):
+        tokens = [r[t] for r in requests]
+        on_gpu = torch.tensor(tokens, dtype=torch.int32, device="cuda:0")
+        a = by_host.step([(s, [tok]) for s, tok in zip(slots_h, tokens)]).clone()
+        b = by_device.step([(s, [0]) for s in slots_d], device_tokens=on_gpu).clone()
+        assert torch.equal(a, b), f"token {t}"
+    check(b[2:3], plain_logits(name, requests[2][:9])[-1:], "bfloat16", "fed from the GPU")
+    if graphs:
+        assert by_device.graph_replays > 0
+    with pytest.raises(StepError, match="device_tokens"):
+        by_device.step([(slots_d[0], [1, 2])], device_tokens=on_gpu[:1])          # not a step of single tokens
+    with pytest.raises(StepError, match="device_tokens"):
+        by_device.step([(s, [0]) for s in slots_d], device_tokens=on_gpu[:2])     # one token short
+    assert [by_device.length(s) for s in slots_d] == [9, 9, 9]
+    by_host.reset()
+    by_device.reset()
+
+
+@pytest.mark.parametrize("graphs", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_a_pass_that_fails_half_way_changes_nothing(dtype, graphs, monkeypatch):
     """A kernel that refuses in the middle of the forward pass (here: the seventh matrix product of

@@ -186,3 +186,68 @@ def test_chunks_cover_every_prompt_once_and_rows_run_out():
         assert all(covered[row] == list(range(n)) for row, n in enumerate(lengths))
     with pytest.raises(bt.GenerationError, match="greater than zero"):
         prefill_chunks([3], 0)
+
+
+def test_decoding_one_step_ahead_feeds_the_right_rows_and_drops_what_a_stop_made_useless():
+    """The decode loop that keeps the host a step behind the GPU, with a scripted engine and
+    sampler (no GPU): every step feeds exactly the rows that can still go on unless their pending
+    token stops them; a row that ends by its length is never fed again; a row that its token ends
+    was fed once more, its slot is closed and its logits row is dropped before the next
+    selection; tokens, order of callbacks and finish reasons are those of the scripted tokens."""
+    import torch
+    from burn_transformers_amd.engine.generate import _decode_ahead
+
+    # what each row will be given, token by token: row 0 stops at its third token (7 is end-of-sequence),
+    # row 1 runs into its own limit of 2, row 2 into max_new_tokens = 5
+    script = {0: [3, 4, 7, 9, 9], 1: [5, 6, 9, 9, 9], 2: [1, 2, 3, 4, 5]}
+    config = bt.GenerationConfig(max_new_tokens=5, eos_token_ids=[7])
+    tracker = GenerationTracker(config, [4, 4, 4], limits=[5, 2, 5])
+
+    class Engine:
+        device = torch.device("cpu")
+
+        def __init__(self):
+            self.fed, self.closed = [], []
+
+        def step(self, entries, device_tokens=None):
+            assert all(tokens == [0] for _, tokens in entries) and device_tokens.numel() == len(entries)
+            self.fed.append([slot for slot, _ in entries])
+            return torch.tensor([[float(slot)] for slot, _ in entries])     # a "logits" row that names its slot
+
+        def close(self, slot):
+            self.closed.append(slot)
+
+    class Sampler:
+        def __init__(self):
+            self.seen, self.steps = [], {row: 0 for row in script}
+
+        def launch(self, logits, rows):
+            assert logits.shape[0] == len(rows)
+            self.seen.append((logits[:, 0].tolist(), list(rows)))
+            self.rows = list(rows)
+
+        def device_ids(self, count):
+            return torch.zeros(count, dtype=torch.int32)
+
+        def result(self):
+            ids = [script[row][self.steps[row]] for row in self.rows]
+            for row in self.rows:
+                self.steps[row] += 1
+            return ids, [-0.5] * len(ids)
+
+    engine, sampler = Engine(), Sampler()
+    slots = [10, 11, 12]
+    open_rows, events = {0, 1, 2}, []
+    first = torch.tensor([[10.0], [11.0], [12.0]])
+    _decode_ahead(engine, sampler, tracker, slots, open_rows, first, [0, 1, 2],
+                  lambda row, token, logp, reason: events.append((row, token, str(reason) if reason else None)))
+    assert [s.token_ids for s in tracker.sequences] == [[3, 4, 7], [5, 6], [1, 2, 3, 4, 5]]
+    assert [str(s.finish_reason) for s in tracker.sequences] == ["EndOfSequence(token_id=7)", "Length", "Length"]
+    # step by step: all three; row 1's second token is its last, so it is not fed; row 0 is fed with
+    # the token that ends it (nobody knew), then is gone; row 2's fifth token is its last
+    assert engine.fed == [[10, 11, 12], [10, 12], [10, 12], [12]]
+    assert engine.closed == [11, 10, 12] and open_rows == set()
+    # every selection saw the logits rows of exactly its live rows, in order
+    assert sampler.seen == [([10.0, 11.0, 12.0], [0, 1, 2]), ([10.0, 11.0, 12.0], [0, 1, 2]), ([10.0, 12.0], [0, 2]),
+                            ([12.0], [2]), ([12.0], [2])]
+    assert [e[:2] for e in events] == [(0, 3), (1, 5), (2, 1), (0, 4), (1, 6), (2, 2), (0, 7), (2, 3), (2, 4), (2, 5)]

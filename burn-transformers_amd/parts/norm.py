@@ -38,7 +38,7 @@ class _KernelNorm(Norm):
         return out
 
     def deferred_possible(self, step, rows):
-        return step.dtype_is_bf16 and K.Normalized.possible(rows, self.width)
+        return step.dtype_is_bf16 and K.Normalized.worth_it(rows, self.width)
 
     def deferred(self, stream, step):
         if stream.pending is not None or not self.deferred_possible(step, stream.x.shape[0]):

@@ -288,6 +288,7 @@ def run_xl(args):
     step_bytes = weight_bytes + args.batch * mean_context * kv_per_token
     achieved = step_bytes / (median / steps) / 1e9
     final_context = PROMPT_LEN + args.warmup + steps + 1
+    from_graphs = engine.graph_replays > 0       # the engine's own choice: a graph only where launching is the limit
 
     prefill_times = prefill_run(engine, vocab, args.repetitions)
     prefill_seconds = statistics.median(prefill_times)
@@ -329,7 +330,7 @@ def run_xl(args):
                    "n_embd": config["n_embd"], "n_head": config["n_head"], "n_inner": config["n_inner"],
                    "vocab_size": vocab, "n_positions": config["n_positions"], "global_batch": args.batch,
                    "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LEN, "final_context": final_context,
-                   "mean_context": round(mean_context, 1), "parallelism": "single GPU", "decode_graphs": True,
+                   "mean_context": round(mean_context, 1), "parallelism": "single GPU", "decode_graphs": from_graphs,
                    "repetitions": args.repetitions, "warmup_repetitions": WARMUP_REPETITIONS},
         "spread": {"min_ms": round(1000.0 * times[0] / steps, 4), "median_ms": round(ms_per_step, 4),
                    "max_ms": round(1000.0 * times[-1] / steps, 4)},

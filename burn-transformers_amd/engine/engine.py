@@ -19,9 +19,14 @@ Steps are replayed from HIP graphs where their shape repeats: a step is hundreds
 and launching them one by one costs the host several microseconds each, more than the short
 kernels of a decode step take to run.  A graph belongs to a shape (tokens, sequences, wanted
 rows, most tokens of one sequence); what differs between steps of one shape (ids, positions,
-block tables, wanted rows) lives in device tables that are filled before each replay.  Decode
-shapes are captured when they come the second time, other shapes the third time.
+block tables, wanted rows) lives in device tables that are filled before each replay.  A step
+that is not replayed runs from its launch list, which a C++ loop walks: with that, and with the
+host kept one step behind the GPU while decoding, a graph pays only where the kernels are so short
+that launching them takes longer than running them (small models, small steps).  So a shape that
+repeats is measured once from its list and captured only if the host was the limit.
 """
+
+import time
 
 import numpy as np
 import torch
@@ -48,7 +53,10 @@ class Engine:
                            model.dtype, model.device, max_slots)
         self.pool = BufferPool(self.device)
         # a mixer that plans work on the host per step cannot be replayed from a graph
-        self.use_graphs = graphs and all(mixer.graph_safe for block in model.blocks for mixer in block.mixers())
+        # graphs: True (capture a repeating shape where a graph pays: see _graph_pays), "always"
+        # (capture every repeating shape) or False
+        self.use_graphs = bool(graphs) and all(mixer.graph_safe for block in model.blocks for mixer in block.mixers())
+        self._graphs_always = graphs == "always"
         # Steps that are not replayed from a graph are kept as launch lists, one per shape, and walked
         # in C++ (kernels.library.Program), if every part of the model only launches kernels
         self.use_programs = programs and getattr(model, "recordable", False)
@@ -61,6 +69,10 @@ class Engine:
         self._pinned_next = 0
         self._graphs = {}                  # shape -> dict(graph, meta, logits, generation), in order of last use
         self._seen = {}                    # shape -> times it came without a graph
+        # shape -> True (its launch list keeps the GPU busy: no graph), False (the host is the limit:
+        # graph), or the measurement under way: (host seconds, start event, end event)
+        self._launch_bound = {}
+        self.graphs_declined = 0           # shapes that were measured and left to their launch lists
         self.steps_run = 0
         self.graph_replays = 0
 
@@ -265,6 +277,8 @@ class Engine:
         if held is not None and held["generation"] != self.pool.generation:
             held = None                                   # a workspace moved: the graph is stale
         if held is None:
+            if self._launch_bound.get(key) is True:       # measured: a graph would gain nothing here
+                return self._run_eager(plan, want_logits=readout)
             # the first times a shape comes it runs eagerly, which also sizes the workspaces
             seen = self._seen.get(key, 0)
             if seen < (1 if plan.decode else 2):
@@ -272,6 +286,8 @@ class Engine:
                     self._seen.clear()
                 self._seen[key] = seen + 1
                 return self._run_eager(plan, want_logits=readout)
+            if self.use_programs and not self._graphs_always and not self._graph_pays(key, plan, readout):
+                return self._latest_logits
             held = self._capture(plan, readout)
             while len(self._graphs) >= _MAX_GRAPHS:
                 self._graphs.pop(next(iter(self._graphs)))
@@ -280,6 +296,40 @@ class Engine:
         held["graph"].replay()
         self.graph_replays += 1
         return held["logits"]
+
+    def _graph_pays(self, key, plan, readout):
+        """Whether the shape should be captured, found out by measuring its launch list once.
+
+        A graph removes the host's cost of launching a step's kernels.  That cost is hidden anyway
+        where the kernels keep the GPU busy for longer than the host needs to launch them (every
+        dependent kernel takes the GPU some microseconds however little it does, and the C++ walk
+        launches one in about three): then a graph gains nothing and costs its capture, a stall of
+        the pipeline, and memory.  So the step that would have been captured runs from its list
+        between two events and the host's time for it is taken; when the shape comes next, the
+        GPU's time is read (one wait, shorter than a capture's) and compared.  Returns False when
+        it ran the step itself (the logits are in ``_latest_logits``)."""
+        probe = self._launch_bound.get(key)
+        if probe is None:
+            if len(self._launch_bound) > 4096:
+                self._launch_bound.clear()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            began = time.perf_counter()
+            start.record()
+            self._latest_logits = self._run_eager(plan, want_logits=readout)
+            end.record()
+            self._launch_bound[key] = (time.perf_counter() - began, start, end)
+            return False
+        if probe is False:
+            return True
+        host_seconds, start, end = probe
+        end.synchronize()
+        gpu_seconds = start.elapsed_time(end) * 1e-3
+        self._launch_bound[key] = gpu_seconds > 1.1 * host_seconds
+        if self._launch_bound[key]:
+            self.graphs_declined += 1
+            self._latest_logits = self._run_eager(plan, want_logits=readout)
+            return False
+        return True
 
     def _capture(self, plan, readout):
         meta = torch.empty(plan.layout.total, dtype=torch.int32, device=self.device)

@@ -111,7 +111,9 @@ def test_48_layers_whole_then_tail_one_by_one(dtype):
     for t in range(64, 96):
         got.append(engine.step([(slot, [ids[t]])]).clone())
     check(torch.cat(got), want, dtype, "the same with its last 32 tokens one by one")
-    assert engine.graph_replays > 0
+    # 343 kernels keep the GPU busy for longer than the C++ walk needs to launch them: the engine
+    # measures that once and leaves the shape to its launch list instead of capturing a graph
+    assert engine.graphs_declined == 1 and engine.graph_replays == 0 and engine.program_runs >= 28
     engine.close(slot)
     engine.cache.ledger.check()
 

@@ -15,6 +15,9 @@ _models = {}
 
 
 def engine_for(name, dtype, max_tokens=2048, gain=1.0, **kw):
+    # these tests are about what graphs replay: every repeating shape is captured, also where the
+    # engine's own choice (graphs=True: only where a graph pays) would leave a shape to its list
+    kw["graphs"] = "always" if kw.get("graphs", True) else False
     key = (name, dtype, gain)
     if key not in _models:
         folder, _, _ = model_folder(name, gain)

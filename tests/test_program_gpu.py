@@ -137,3 +137,23 @@ def test_host_time_of_a_listed_step_is_a_fraction_of_the_direct_one():
     print(f"host time of a 64-token step of a 3-layer model: {seconds[True] * 1e6:.0f} us from a launch list, "
           f"{seconds[False] * 1e6:.0f} us call by call")
     assert seconds[True] < 0.7 * seconds[False]
+
+
+def test_a_small_model_whose_launches_outlast_its_kernels_is_captured():
+    """The engine's own choice (graphs=True): a repeating shape is measured once from its launch
+    list; here the kernels are so short that launching them takes the host longer than they run,
+    so the shape is captured and replayed (the opposite case, a model whose kernels outlast their
+    launches, is the 48-layer test of test_depth_gpu.py)."""
+    model = model_for("A", "bfloat16")
+    engine = bt.Engine(model, max_tokens=256)
+    assert engine.use_graphs and engine.use_programs
+    ids = prompts_for("A", [40], seed=86)[0]
+    slot = engine.open()
+    rows = [engine.step([(slot, ids[:8])], want=[list(range(8))]).clone()]
+    for t in range(8, 40):
+        rows.append(engine.step([(slot, [ids[t]])]).clone())
+    # the shape's first step records its list, the second runs from it and is timed, the third reads the
+    # timing, captures and replays
+    assert engine.graphs_declined == 0 and engine.graph_replays == 32 - 2
+    want = plain_logits("A", ids)
+    assert float((torch.cat(rows).cpu().double() - want).abs().max()) <= tolerance("bfloat16", want)

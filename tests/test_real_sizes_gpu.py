@@ -139,7 +139,7 @@ def test_last_32_tokens_one_by_one_up_to_the_position_limit(dtype):
     for t in range(head, len(ids)):
         got.append(engine.step([(slot, [ids[t]])]).clone())
     check(torch.cat(got), plain_rows(ids, [0, 500, head - 1] + list(range(head, len(ids)))), dtype, "tail of 1,024")
-    assert engine.graph_replays > 0
+    assert engine.graph_replays + engine.program_runs > 0
     engine.close(slot)
 
 

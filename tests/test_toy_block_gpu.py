@@ -190,7 +190,7 @@ def test_blocks_with_other_roles_no_mixer_and_a_turning_mixer(dtype, tmp_path):
         model = bt.load_model(str(tmp_path), dtype=dtype)
         assert [len(block.mixers()) for block in model.blocks] == [1, 0]
         assert model.blocks[1].cache_needs() == (None, None) and model.cache_entries == 2
-        engine = bt.Engine(model, max_tokens=1024)
+        engine = bt.Engine(model, max_tokens=1024, graphs="always")
         assert engine.use_graphs
         w = {k: v.double() for k, v in stored.items()}
         gen = torch.Generator().manual_seed(4)

@@ -139,7 +139,7 @@ def test_routed_feed_forward_and_sinusoid_positions(dtype, tmp_path):
         config = RoutedConfig()
         stored = bt.write_random_model(str(tmp_path), config.to_dict(), seed=5)
         model = bt.load_model(str(tmp_path), dtype=dtype)
-        engine = bt.Engine(model, max_tokens=512)
+        engine = bt.Engine(model, max_tokens=512, graphs="always")
         assert engine.use_graphs
         w = {k: v.double() for k, v in stored.items()}
         gen = torch.Generator().manual_seed(1)

@@ -77,7 +77,7 @@ def test_layers_with_windows_give_blocks_back_and_read_nothing_that_is_gone(dtyp
         _, tensors = bt.random_tensors(CONFIG, 9)
         tensors = {k: (v * 5.0 if v.dim() == 2 else v).to(torch.bfloat16).float() for k, v in tensors.items()}
         model = bt.model_from_tensors(CONFIG, tensors, dtype=dtype, device="cuda:0")
-        engine = bt.Engine(model, max_tokens=64 * 17)
+        engine = bt.Engine(model, max_tokens=64 * 17, graphs="always")
         cache, ledger = engine.cache, engine.cache.ledger
         # three groups: every key (layer 0), the last 70 (layers 1 and 3), the last 200 (layer 2)
         assert sorted(ledger.windows) == [0, 70, 200] and [g.entries for g in cache.kv_groups] == [1, 2, 1]

@@ -582,6 +582,59 @@ def test_prefill_attention_every_query_finds_its_one_key(dtype, q_heads, kv_head
         f"query row {worst} (position {int(case.tok_pos[worst])} of sequence {int(case.tok_seq[worst])}) is off by {float(error.max())}"
 
 
+@pytest.mark.parametrize("dtype,hd,window,totals,counts", [
+    ("bfloat16", 64, 100, [700, 333], [517, 70]),
+    ("bfloat16", 32, 64, [300, 200], [300, 1]),
+    ("bfloat16", 64, 33, [500, 90, 41], [1, 1, 1]),            # a decode step
+    ("float32", 64, 100, [700, 333], [517, 70]),
+    ("float32", 48, 33, [500, 90, 41], [1, 1, 1]),
+])
+def test_attention_at_the_edge_of_a_window(dtype, hd, window, totals, counts):
+    """A query with a window of w sees keys pos - w + 1 ... pos.  Every even query is given one key
+    that takes all the weight at the first position it still sees, every odd query at the position
+    just before, which it must not see: counted in, that key would turn the output into its value
+    row; left out, the output is the softmax over the window.  An off-by-one at either edge shows
+    as an error of the size of a value, in the kernels for prompts and for single tokens."""
+    dt = DTYPES[dtype]
+    q_heads = kv_heads = 2
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=41, poison=True)
+    q = torch.zeros(case.n_tokens, q_heads * hd)
+    row, inside, outside = 0, 0, 0
+    for s, (total, count) in enumerate(zip(totals, counts)):
+        keys = case.k_rows[s].float().view(total, kv_heads, hd)
+        keys = keys / keys.norm(dim=-1, keepdim=True)
+        case.k_rows[s] = keys.reshape(total, kv_heads * hd).to(dt)
+        stored = case.k_rows[s].float().view(total, kv_heads, hd)
+        for i in range(count):
+            pos = total - count + i
+            target = pos - window + 1 if row % 2 == 0 else pos - window
+            if target >= 0:
+                q[row] = stored[target].reshape(-1)
+                inside, outside = inside + (row % 2 == 0), outside + (row % 2 == 1)
+            else:
+                q[row] = stored[pos].reshape(-1)
+            row += 1
+    assert inside > 0 and outside > 0
+    seq = torch.cat([torch.full((t,), s, dtype=torch.int32) for s, t in enumerate(totals)]).to(DEV)
+    pos = torch.cat([torch.arange(t, dtype=torch.int32) for t in totals]).to(DEV)
+    K.kv_copy(torch.cat(case.k_rows).to(DEV), torch.cat(case.v_rows).to(DEV), seq, pos, case.view(), True)
+    q = q.to(dt).to(DEV)
+    scale = 60.0
+    want = case.reference(q, q_heads, scale, window)
+    decode = max(counts) == 1
+    impls = (["mfma"] if dtype == "bfloat16" else ["tiled"]) + ["plain"]
+    for impl in impls:
+        for as_decode in ([False, True] if decode and impl == "mfma" else [decode]):
+            out = torch.full((case.n_tokens, q_heads * hd), float("nan"), dtype=dt, device=DEV)
+            args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                                    q_heads, len(totals), max(counts), scale, window)
+            K.attention(args, dt, decode=as_decode, impl=impl)
+            error = (out.detach().cpu().double() - want).abs().max(dim=1).values
+            worst = int(error.argmax())
+            assert float(error.max()) < (3e-2 if dtype == "bfloat16" else 1e-4), \
+                f"{impl} (decode kernel: {as_decode}): query row {worst} at position {int(case.tok_pos[worst])} is off by {float(error.max())}"
+
+
 @pytest.mark.parametrize("dtype,hd,window", [("bfloat16", 64, 0), ("bfloat16", 32, 0), ("bfloat16", 64, 3000),
                                              ("float32", 64, 0), ("float32", 112, 0), ("float32", 48, 1500)])
 def test_attention_decode_in_runs(dtype, hd, window):

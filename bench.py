@@ -1,7 +1,7 @@
 """Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
-                    [--repetitions 10] [--workload xl|small|medium|sweep] [--no-points] [--no-kernels]
+                    [--repetitions 10] [--workload xl|small|medium|sweep] [--no-points] [--no-kernels] [--no-own]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
 sequences, prefilled with 512 synthetic tokens each, is decoded towards 1,024.  A step is one
@@ -301,7 +301,7 @@ def run_xl(args):
     if not args.no_kernels:
         kernels["decode"] = decode_kernels(engine, args.batch, vocab, config, args.dtype, int(mean_context))
         kernels["prefill"] = prefill_kernels(engine, vocab, config, args.dtype)
-    if args.dtype == "bf16" and K.library_products() is not None:
+    if args.dtype == "bf16" and K.library_products() is not None and not args.no_own:
         # the same step with every product on this package's own kernels
         held = dict(K._library_state)
         K._library_state.update(tried=True, lib=None)
@@ -464,6 +464,7 @@ def main():
     parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep"], default="xl")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     parser.add_argument("--no-kernels", action="store_true", help="skip the classes of kernels on their own")
+    parser.add_argument("--no-own", action="store_true", help="skip the prefill on this package's own product kernels")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this library")

@@ -278,12 +278,6 @@ class _Recording:
         return False
 
 
-def recording():
-    """True while kernel calls are being kept in a launch list instead of being launched: a part
-    that does anything but call this module's kernels cannot be recorded."""
-    return _recorder[0] is not None
-
-
 _held_stream = [None]
 
 

@@ -80,14 +80,27 @@ attention_f32_kernel(AttnArgs a) {
       vreg[j] = *reinterpret_cast<const floatx4*>(values + base + (int64_t)at * 4);
     }
   };
-  auto stage = [&]() __attribute__((always_inline)) {
+  // Positions behind the tile's last query hold no token of this step and may hold anything, NaN
+  // included (a block that another sequence used before), and 0 * NaN is NaN: their values are
+  // replaced by zero here, once per block and only in the sequence's last block, so that the
+  // multiplications below need no test of their own (a select beside every FMA cost the value
+  // phase half its time).  Everything at or before the last query is a token of this sequence.
+  auto stage = [&](int block) __attribute__((always_inline)) {
+    const int beyond = last_pos - block * BT_KV_BLOCK;        // positions of the block above this hold no token
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
       int piece = tid + 256 * j;
       if (piece < pieces) {
         int row = piece / (hd / 4), c4 = piece % (hd / 4);
         *reinterpret_cast<floatx4*>(ks + row * (hd + 4) + c4 * 4) = kreg[j];
-        *reinterpret_cast<floatx4*>(vs + piece * 4) = vreg[j];
+        floatx4 v = vreg[j];
+        if (beyond < BT_KV_BLOCK - 1) {                       // (the same for the whole work-group)
+          int first = (piece / hd) * 4;                       // the piece holds positions first .. first + 3 of one channel
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (first + r > beyond) v[r] = 0.f;
+        }
+        *reinterpret_cast<floatx4*>(vs + piece * 4) = v;
       }
     }
   };
@@ -108,7 +121,7 @@ attention_f32_kernel(AttnArgs a) {
   fetch(first_block);
   for (int block = first_block; block <= last_block; ++block) {
     __syncthreads();                                          // the previous block's LDS is no longer read
-    stage();
+    stage(block);
     if (block < last_block) fetch(block + 1);                 // in flight while this block is worked on
     __syncthreads();
     float rescale[F32_WAVE_QUERIES];
@@ -159,7 +172,10 @@ attention_f32_kernel(AttnArgs a) {
       for (int i = 0; i < F32_WAVE_QUERIES; ++i)
 #pragma unroll
         for (int j = 0; j < CPT; ++j) acc[i][j] *= rescale[i];
-      // values: channel lane (+ 64) of four keys at a time
+      // values: channel lane (+ 64) of four keys at a time.  Unrolled by two: measured at 2 x 1,024
+      // tokens of 25 heads of 64, 461 / 445 / 546 us a layer unrolled by 1 / 2 / 4 (whole, the
+      // compiler hoists every read above the arithmetic and spills: 1,900 us)
+#pragma unroll 2
       for (int k4 = 0; k4 < BT_KV_BLOCK / 4; ++k4) {
         float4 v4[CPT];
 #pragma unroll
@@ -173,12 +189,11 @@ attention_f32_kernel(AttnArgs a) {
           float4 p4 = *reinterpret_cast<const float4*>(ps + (my_q + i) * BT_KV_BLOCK + k4 * 4);
 #pragma unroll
           for (int j = 0; j < CPT; ++j) {
-            // a position that holds no token yet may hold anything, NaN included, and 0 * NaN is
-            // NaN: what is not seen is not multiplied
-            acc[i][j] = p4.x != 0.f ? fmaf(p4.x, v4[j].x, acc[i][j]) : acc[i][j];
-            acc[i][j] = p4.y != 0.f ? fmaf(p4.y, v4[j].y, acc[i][j]) : acc[i][j];
-            acc[i][j] = p4.z != 0.f ? fmaf(p4.z, v4[j].z, acc[i][j]) : acc[i][j];
-            acc[i][j] = p4.w != 0.f ? fmaf(p4.w, v4[j].w, acc[i][j]) : acc[i][j];
+            // (values of positions that hold no token were zeroed when the block was staged)
+            acc[i][j] = fmaf(p4.x, v4[j].x, acc[i][j]);
+            acc[i][j] = fmaf(p4.y, v4[j].y, acc[i][j]);
+            acc[i][j] = fmaf(p4.z, v4[j].z, acc[i][j]);
+            acc[i][j] = fmaf(p4.w, v4[j].w, acc[i][j]);
           }
         }
       }

@@ -312,6 +312,12 @@ class Engine:
         if probe is None:
             if len(self._launch_bound) > 4096:
                 self._launch_bound.clear()
+            if key not in self._programs and self._seen.get(key, 0) < 8:
+                # the shape has no list yet (its first step made a workspace grow): this step would be
+                # launched from Python and say nothing about the list; it records, the next one is measured
+                self._seen[key] = self._seen.get(key, 0) + 1
+                self._latest_logits = self._run_eager(plan, want_logits=readout)
+                return False
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             began = time.perf_counter()
             start.record()

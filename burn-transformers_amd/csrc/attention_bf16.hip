@@ -304,19 +304,37 @@ attention_prefill_kernel(AttnArgs a) {
   }
 }
 
-// A whole block of 64 keys at once, for the kernel that has it in LDS: the same steps as
-// attend_tile with half as many maxima, exchanges between lanes and rescaling tests per key,
-// and four independent score blocks for the scheduler to interleave (one wave is often alone
-// on its SIMD here, so nothing else hides the latency of a dependent chain).
+// The largest of three in one instruction.  (fmaxf first passes every operand that comes out of
+// a matrix instruction through an instruction of its own, to quieten a signalling NaN.)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// A whole block of 64 keys at once, for the kernel that has it in LDS.  The softmax's own
+// arithmetic sets that kernel's time, so this form spends as few vector instructions per score
+// as it can:
+//   * a lane looks at its OWN sixteen scores of a query only; the four lanes of a query compare
+//     notes (two exchanges between lanes, and the rescaling of every sum) only when some lane of
+//     the wave has a score more than RESCALE_SLACK powers of two above the query's running
+//     maximum, which after a sequence's first blocks is rare;
+//   * the sums of the probabilities come from the matrix unit: one more product with a tile of
+//     ones adds, for every query, exactly the bfloat16 probabilities that the output rows are
+//     made of, and leaves the whole sum in every lane of the query (rows[nq][*] all equal), so
+//     nothing is added up lane by lane, during the walk or after it.
+//   `masked` (the same for the whole wave) says that some query of the wave does not see the
+//   whole block; both kinds of block run the same instructions but for the replacement of the
+//   excluded scores, so the compiler keeps every running sum in one place.
 struct BlockOperands {
   bf16x8 k[4][NKS];
-  bf16x4 v[ND][4];
+  bf16x8 v[ND][2];   // [block of 16 channels][half of the block's positions]: see SHARED_V_BYTES
 };
 
-template <int NQ, bool MASKED>
-__device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, int valid_end,
+template <int NQ>
+__device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, int valid_end, bool masked,
                                              const int (&qpos)[NQ], float c, const bf16x8 (&q)[NQ][NKS],
-                                             floatx4 (&o)[NQ][ND], float (&m)[NQ], float (&l)[NQ]) {
+                                             floatx4 (&o)[NQ][ND], float (&m)[NQ], floatx4 (&rows)[NQ]) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
   floatx4 s[NQ][4];
 #pragma unroll
@@ -330,32 +348,41 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
       s[nq][t] = acc;
     }
   }
-  float m_new[NQ];
-  bool behind = false;
+  if (masked) {
 #pragma unroll
-  for (int nq = 0; nq < NQ; ++nq) {
-    if (MASKED) {
+    for (int nq = 0; nq < NQ; ++nq) {
       const int qp = qpos[nq];
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) s[nq][t][r] = kb + 16 * t + 4 * g + r <= qp ? s[nq][t][r] : -INFINITY;
     }
-    float tile_max = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-      tile_max = fmaxf(tile_max, fmaxf(fmaxf(s[nq][t][0], s[nq][t][1]), fmaxf(s[nq][t][2], s[nq][t][3])));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-    m_new[nq] = fmaxf(m[nq], tile_max * c);
-    behind = behind || m_new[nq] > m[nq] + RESCALE_SLACK;
   }
-  if (__builtin_amdgcn_ballot_w64(behind) != 0) {
+  float own[NQ];
+  bool behind = false;
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    float top = max3(s[nq][0][0], s[nq][0][1], s[nq][0][2]);
+    top = max3(top, s[nq][0][3], s[nq][1][0]);
+    top = max3(top, s[nq][1][1], s[nq][1][2]);
+    top = max3(top, s[nq][1][3], s[nq][2][0]);
+    top = max3(top, s[nq][2][1], s[nq][2][2]);
+    top = max3(top, s[nq][2][3], s[nq][3][0]);
+    top = max3(top, s[nq][3][1], s[nq][3][2]);
+    own[nq] = fmaxf(top, s[nq][3][3]) * c;
+    behind = behind || own[nq] > m[nq] + RESCALE_SLACK;   // true for a query's first block: m starts at -inf
+  }
+  if (__builtin_amdgcn_ballot_w64(behind) != 0) {   // the same for the whole wave: a scalar branch
 #pragma unroll
     for (int nq = 0; nq < NQ; ++nq) {
-      float alpha = m_new[nq] == -INFINITY ? 1.f : exp2f(m[nq] - m_new[nq]);
-      m[nq] = m_new[nq];
-      l[nq] *= alpha;
+      float top = own[nq];
+      top = fmaxf(top, __shfl_xor(top, 16, 64));
+      top = fmaxf(top, __shfl_xor(top, 32, 64));
+      const float m_new = fmaxf(m[nq], top);
+      const float alpha = m_new == -INFINITY ? 1.f : exp2f(m[nq] - m_new);
+      m[nq] = m_new;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) rows[nq][r] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -366,31 +393,32 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
     const float m_use = m[nq] == -INFINITY ? 0.f : m[nq];
-    float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float p = __builtin_amdgcn_exp2f(fmaf(s[nq][t][r], c, -m_use));
-        psum += p;
-        pop[nq][t >> 1][4 * (t & 1) + r] = (bf16_t)p;
-      }
-    l[nq] += psum;
+      for (int r = 0; r < 4; ++r)
+        pop[nq][t >> 1][4 * (t & 1) + r] = (bf16_t)__builtin_amdgcn_exp2f(fmaf(s[nq][t][r], c, -m_use));
   }
-  const bool ragged = MASKED && kb + 64 > valid_end;
+  const bf16_t one = (bf16_t)1.0f;
+  const bf16x8 ones = {one, one, one, one, one, one, one, one};
+#pragma unroll
+  for (int half = 0; half < 2; ++half)
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq)
+      rows[nq] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pop[nq][half], rows[nq], 0, 0, 0);
+  const bool ragged = masked && kb + 64 > valid_end;
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt) {
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      bf16x4 v0 = blk.v[dt][2 * half], v1 = blk.v[dt][2 * half + 1];
+      bf16x8 vop = blk.v[dt][half];
       if (ragged) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          if (kb + 32 * half + 4 * g + r >= valid_end) v0[r] = (bf16_t)0.f;
-          if (kb + 32 * half + 16 + 4 * g + r >= valid_end) v1[r] = (bf16_t)0.f;
+          if (kb + 32 * half + 4 * g + r >= valid_end) vop[r] = (bf16_t)0.f;
+          if (kb + 32 * half + 16 + 4 * g + r >= valid_end) vop[4 + r] = (bf16_t)0.f;
         }
       }
-      bf16x8 vop = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
 #pragma unroll
       for (int nq = 0; nq < NQ; ++nq)
         o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[nq][half], o[nq][dt], 0, 0, 0);
@@ -407,11 +435,16 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 // pull (about 25 GB/s): the four or eight waves asked for the same bytes four or eight times.
 //   keys:   row r (128 bytes) keeps its 16-byte chunk c at c ^ ((r >> 1) & 7): the 16 lanes of
 //           a ds_read_b128 that read one chunk of 16 consecutive rows then hit different banks;
-//   values: the 512 bytes of a group of four positions are followed by 128 bytes of padding, so
-//           that the groups g and g + 1 a ds_read_b64 touches together lie in different banks.
+//   values: in the order of the MFMA operand.  A lane (channel i of a block of 16, group g of the
+//           lanes) multiplies, for half h of the block's positions, the eight values of positions
+//           32 h + 4 g + 0..3 and 32 h + 16 + 4 g + 0..3 of its channel: those 16 bytes lie
+//           together at ((4 h + g) * 64 + channel) * 16, so an operand is ONE ds_read_b128 and
+//           the 16 lanes of a group read 256 consecutive bytes.  (The cache keeps four
+//           consecutive positions of a channel together: a thread brings the two groups of four
+//           positions of ONE channel that belong to one operand, eight bytes each, and stores
+//           them as one 16-byte piece, a wave 1,024 consecutive bytes.)
 #define SHARED_K_BYTES (64 * 128)
-#define SHARED_V_GROUP 640
-#define SHARED_V_BYTES (16 * SHARED_V_GROUP)
+#define SHARED_V_BYTES (64 * 128)
 #define SHARED_STAGE (SHARED_K_BYTES + SHARED_V_BYTES)
 
 // The KEYS of a tile are divided between two sets of four waves:
@@ -424,8 +457,16 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 // every SIMD has two waves at work all the time instead of one for most of it.  The tiles are
 // numbered latest first over the whole grid, so that the short ones fill in behind the long
 // ones.  Measured at 25 heads: 2 x 1,024 tokens 29.3 -> 27.3 us, 2,048 tokens 50.2 -> 43.2 us,
-// 4 chunks of 256 tokens behind 768 28.4 -> 21.8 us; what is left is the softmax's own
-// arithmetic (32 exponentials per lane and block at a quarter of the VALU rate).
+// 4 chunks of 256 tokens behind 768 28.4 -> 21.8 us.  With the leaner softmax of block_output
+// (maxima per lane, sums from the matrix unit, values in LDS in operand order): 24.5, 38.5 and
+// 20.3 us, and 8,192 tokens of one sequence 503 -> 445 us (480 TFLOP/s).  What the time goes to
+// then, measured by leaving parts out at 8,192 tokens: with no loads from memory, no writes to
+// LDS and no barrier 290 to 320 us are left, which is the waves' own instruction streams (two
+// waves per SIMD, each issuing some 115 vector instructions, 32 exponentials at a quarter of
+// the rate and 36 matrix instructions per block); the loads cost 80 us, the writes 28, the
+// barrier 39.  Keeping three turns in LDS, so that operands are read a turn ahead and nobody
+// waits at the barrier, and reading the block table a turn ahead were both tried and gained
+// nothing: the cost of those parts is their instructions, not their waiting.
 #define SPLIT_TURN (2 * SHARED_STAGE)
 #define SPLIT_LDS_BYTES (2 * SPLIT_TURN)
 
@@ -463,8 +504,8 @@ attention_prefill_split_kernel(AttnArgs a) {
 
   int qpos[PREFILL_NQ], tok[PREFILL_NQ];
   bf16x8 q[PREFILL_NQ][NKS];
-  floatx4 o[PREFILL_NQ][ND];
-  float m[PREFILL_NQ], l[PREFILL_NQ];
+  floatx4 o[PREFILL_NQ][ND], rows[PREFILL_NQ];   // rows[nq][*]: the sum of query nq's probabilities
+  float m[PREFILL_NQ];
 #pragma unroll
   for (int nq = 0; nq < PREFILL_NQ; ++nq) {
     int qi = q0 + nq * 16 + i16;
@@ -476,8 +517,8 @@ attention_prefill_split_kernel(AttnArgs a) {
       q[nq][ks] = load_bf16x8(Q + (int64_t)tok[nq] * a.ldq + head * HD + ks * 32 + g * 8);
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt) o[nq][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    rows[nq] = floatx4{0.f, 0.f, 0.f, 0.f};
     m[nq] = -INFINITY;
-    l[nq] = 0.f;
   }
   const int last = q0 + PREFILL_QUERIES_PER_WAVE < count ? q0 + PREFILL_QUERIES_PER_WAVE : count;
   const int hi = active ? start + last : 0;     // one past the position of this wave's last query
@@ -487,6 +528,7 @@ attention_prefill_split_kernel(AttnArgs a) {
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
 
+  typedef __attribute__((__vector_size__(2 * sizeof(int)))) int int2v;
   int4v kreg[2], vreg[2];
   auto fetch = [&](int turn) {
 #pragma unroll
@@ -495,16 +537,19 @@ attention_prefill_split_kernel(AttnArgs a) {
       if (block_index >= n_blocks) block_index = n_blocks - 1;     // (read again, never multiplied)
       int64_t plane = tile_plane(a, seq, kv_head, block_index * BT_KV_BLOCK);
       kreg[b] = *reinterpret_cast<const int4v*>(keys + plane + tid * 8);
-      vreg[b] = *reinterpret_cast<const int4v*>(values + plane + tid * 8);
+      // the thread's values: one channel, the two groups of four positions that one operand holds
+      const bf16_t* mine = values + plane + ((tid >> 8) * 8 + ((tid >> 6) & 3)) * (4 * HD) + (tid & 63) * 4;
+      const int2v low = *reinterpret_cast<const int2v*>(mine), high = *reinterpret_cast<const int2v*>(mine + 16 * HD);
+      vreg[b] = int4v{low[0], low[1], high[0], high[1]};
     }
   };
   auto stash = [&](unsigned char* turn_base) {
-    const int row = tid >> 3, chunk = tid & 7, grp = tid >> 5, within = tid & 31;
+    const int row = tid >> 3, chunk = tid & 7;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       unsigned char* stage = turn_base + b * SHARED_STAGE;
       *reinterpret_cast<int4v*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4)) = kreg[b];
-      *reinterpret_cast<int4v*>(stage + SHARED_K_BYTES + grp * SHARED_V_GROUP + within * 16) = vreg[b];
+      *reinterpret_cast<int4v*>(stage + SHARED_K_BYTES + tid * 16) = vreg[b];   // ((4 h + g) * 64 + channel) * 16
     }
   };
   fetch(0);
@@ -526,16 +571,12 @@ attention_prefill_split_kernel(AttnArgs a) {
           blk.k[kt][ks] = *reinterpret_cast<const bf16x8*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
         }
 #pragma unroll
-      for (int dt = 0; dt < ND; ++dt) {
-        const unsigned char* column = stage + SHARED_K_BYTES + (dt * 16 + i16) * 8;
+      for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
-        for (int quarter = 0; quarter < 4; ++quarter)
-          blk.v[dt][quarter] = *reinterpret_cast<const bf16x4*>(column + (4 * quarter + g) * SHARED_V_GROUP);
-      }
-      if (kb + 64 <= whole_until)
-        attend_block<PREFILL_NQ, false>(blk, kb, valid_end, qpos, c, q, o, m, l);
-      else
-        attend_block<PREFILL_NQ, true>(blk, kb, valid_end, qpos, c, q, o, m, l);
+        for (int half = 0; half < 2; ++half)
+          blk.v[dt][half] = *reinterpret_cast<const bf16x8*>(stage + SHARED_K_BYTES +
+                                                             ((4 * half + g) * 64 + dt * 16 + i16) * 16);
+      attend_block<PREFILL_NQ>(blk, kb, valid_end, kb + 64 > whole_until, qpos, c, q, o, m, rows);
     }
     if (more) stash(split_lds + ((t + 1) & 1) * SPLIT_TURN);
     __syncthreads();   // turn t + 1 is in place, and everyone is done with turn t before it is overwritten
@@ -549,7 +590,7 @@ attention_prefill_split_kernel(AttnArgs a) {
     for (int nq = 0; nq < PREFILL_NQ; ++nq) {
       const int k0 = nq * PER_QUERY;
       hand[((k0 + 0) * PREFILL_WAVES + wave) * 64 + lane] = m[nq];
-      hand[((k0 + 1) * PREFILL_WAVES + wave) * 64 + lane] = l[nq];
+      hand[((k0 + 1) * PREFILL_WAVES + wave) * 64 + lane] = rows[nq][0];
 #pragma unroll
       for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -567,9 +608,7 @@ attention_prefill_split_kernel(AttnArgs a) {
     const float top = fmaxf(m[nq], m_other);                       // (the maxima are kept in powers of two)
     const float mine = m[nq] == -INFINITY ? 0.f : exp2f(m[nq] - top);
     const float theirs = m_other == -INFINITY ? 0.f : exp2f(m_other - top);
-    float total = l[nq] * mine + l_other * theirs;
-    total += __shfl_xor(total, 16, 64);
-    total += __shfl_xor(total, 32, 64);
+    const float total = rows[nq][0] * mine + l_other * theirs;   // (whole sums: see attend_block)
     float inv = total > 0.f ? 1.0f / total : 0.f;
     if (qpos[nq] < 0) continue;
 #pragma unroll

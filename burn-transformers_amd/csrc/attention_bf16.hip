@@ -70,6 +70,27 @@ __device__ __forceinline__ void load_tile(TileOperands& t, const bf16_t* __restr
   }
 }
 
+// The online softmax of both forms below works on exponents, x = score * c - (the query's running
+// maximum, which may lag: RESCALE_SLACK), computed by the one FMA that the exponential needs
+// anyway.  A lane looks at its OWN exponents only; the four lanes of a query compare notes, and
+// every sum is rescaled, only when some lane of the wave has an exponent above RESCALE_SLACK (or
+// a query meets its first key), which after a sequence's first tiles is rare.  (The maxima are
+// taken of the FMA's results, not of the scores as the matrix unit leaves them: those the
+// compiler would first pass through an instruction each to quieten a signalling NaN, and an
+// instruction written by hand instead is not seen by the compiler's bookkeeping of the wait
+// between a matrix instruction and the first read of its result: that was a real wrong result.)
+//   m: the running maximum (-inf before the first key); top: the largest exponent of the tile
+//   among the query's four lanes.  Returns what to take off the tile's exponents; `alpha` is what
+//   the running sums are to be multiplied with.
+__device__ __forceinline__ float raise_maximum(float& m, float top, float& alpha) {
+  const bool fresh = m == -INFINITY;        // the exponents were taken against 0 then
+  const bool nothing = top == -INFINITY;    // every key of the tile is excluded for this query
+  const float delta = fresh ? (nothing ? 0.f : top) : fmaxf(top, 0.f);
+  alpha = fresh ? 1.f : exp2f(-delta);      // (sums of a fresh query are zero)
+  m = fresh ? (nothing ? -INFINITY : top) : m + delta;
+  return delta;
+}
+
 // The running maximum of a query may lag behind the true one by up to this many powers of two
 // before the sums are rescaled: probabilities then reach at most 2^RESCALE_SLACK instead of 1,
 // which 32-bit sums and bfloat16 operands (a relative format) carry as well, and the rescaling
@@ -101,7 +122,7 @@ __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, in
       s[nq][t] = acc;
     }
   }
-  float m_new[NQ];
+  float own[NQ];
   bool behind = false;
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
@@ -116,19 +137,28 @@ __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, in
           s[nq][t][r] = seen ? s[nq][t][r] : -INFINITY;
         }
     }
-    float tile_max = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
-                           fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-    m_new[nq] = fmaxf(m[nq], tile_max * c);
-    behind = behind || m_new[nq] > m[nq] + RESCALE_SLACK;   // true for the first tile: m starts at -inf
+    const float m_use = m[nq] == -INFINITY ? 0.f : m[nq];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[nq][t][r] = fmaf(s[nq][t][r], c, -m_use);
+    own[nq] = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
+                    fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
+    behind = behind || own[nq] > (m[nq] == -INFINITY ? -INFINITY : RESCALE_SLACK);
   }
   if (__builtin_amdgcn_ballot_w64(behind) != 0) {   // the same for the whole wave: a scalar branch
 #pragma unroll
     for (int nq = 0; nq < NQ; ++nq) {
-      float alpha = m_new[nq] == -INFINITY ? 1.f : exp2f(m[nq] - m_new[nq]);
-      m[nq] = m_new[nq];
+      float top = own[nq];
+      top = fmaxf(top, __shfl_xor(top, 16, 64));
+      top = fmaxf(top, __shfl_xor(top, 32, 64));
+      float alpha;
+      const float delta = raise_maximum(m[nq], top, alpha);
       l[nq] *= alpha;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[nq][t][r] -= delta;
 #pragma unroll
       for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -138,13 +168,12 @@ __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, in
   bf16x8 pop[NQ];
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
-    const float m_use = m[nq] == -INFINITY ? 0.f : m[nq];
     float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float p = __builtin_amdgcn_exp2f(fmaf(s[nq][t][r], c, -m_use));
+        float p = __builtin_amdgcn_exp2f(s[nq][t][r]);
         psum += p;
         pop[nq][4 * t + r] = (bf16_t)p;
       }
@@ -304,21 +333,10 @@ attention_prefill_kernel(AttnArgs a) {
   }
 }
 
-// The largest of three in one instruction.  (fmaxf first passes every operand that comes out of
-// a matrix instruction through an instruction of its own, to quieten a signalling NaN.)
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
-
 // A whole block of 64 keys at once, for the kernel that has it in LDS.  The softmax's own
 // arithmetic sets that kernel's time, so this form spends as few vector instructions per score
 // as it can:
-//   * a lane looks at its OWN sixteen scores of a query only; the four lanes of a query compare
-//     notes (two exchanges between lanes, and the rescaling of every sum) only when some lane of
-//     the wave has a score more than RESCALE_SLACK powers of two above the query's running
-//     maximum, which after a sequence's first blocks is rare;
+//   * maxima per lane, lanes exchanging theirs only when sums are rescaled (raise_maximum);
 //   * the sums of the probabilities come from the matrix unit: one more product with a tile of
 //     ones adds, for every query, exactly the bfloat16 probabilities that the output rows are
 //     made of, and leaves the whole sum in every lane of the query (rows[nq][*] all equal), so
@@ -362,15 +380,17 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
   bool behind = false;
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
-    float top = max3(s[nq][0][0], s[nq][0][1], s[nq][0][2]);
-    top = max3(top, s[nq][0][3], s[nq][1][0]);
-    top = max3(top, s[nq][1][1], s[nq][1][2]);
-    top = max3(top, s[nq][1][3], s[nq][2][0]);
-    top = max3(top, s[nq][2][1], s[nq][2][2]);
-    top = max3(top, s[nq][2][3], s[nq][3][0]);
-    top = max3(top, s[nq][3][1], s[nq][3][2]);
-    own[nq] = fmaxf(top, s[nq][3][3]) * c;
-    behind = behind || own[nq] > m[nq] + RESCALE_SLACK;   // true for a query's first block: m starts at -inf
+    const float m_use = m[nq] == -INFINITY ? 0.f : m[nq];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[nq][t][r] = fmaf(s[nq][t][r], c, -m_use);
+    float top = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      top = fmaxf(top, fmaxf(fmaxf(s[nq][t][0], s[nq][t][1]), fmaxf(s[nq][t][2], s[nq][t][3])));
+    own[nq] = top;
+    behind = behind || top > (m[nq] == -INFINITY ? -INFINITY : RESCALE_SLACK);
   }
   if (__builtin_amdgcn_ballot_w64(behind) != 0) {   // the same for the whole wave: a scalar branch
 #pragma unroll
@@ -378,9 +398,12 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
       float top = own[nq];
       top = fmaxf(top, __shfl_xor(top, 16, 64));
       top = fmaxf(top, __shfl_xor(top, 32, 64));
-      const float m_new = fmaxf(m[nq], top);
-      const float alpha = m_new == -INFINITY ? 1.f : exp2f(m[nq] - m_new);
-      m[nq] = m_new;
+      float alpha;
+      const float delta = raise_maximum(m[nq], top, alpha);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[nq][t][r] -= delta;
 #pragma unroll
       for (int r = 0; r < 4; ++r) rows[nq][r] *= alpha;
 #pragma unroll
@@ -392,12 +415,10 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
   bf16x8 pop[NQ][2];
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
-    const float m_use = m[nq] == -INFINITY ? 0.f : m[nq];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        pop[nq][t >> 1][4 * (t & 1) + r] = (bf16_t)__builtin_amdgcn_exp2f(fmaf(s[nq][t][r], c, -m_use));
+      for (int r = 0; r < 4; ++r) pop[nq][t >> 1][4 * (t & 1) + r] = (bf16_t)__builtin_amdgcn_exp2f(s[nq][t][r]);
   }
   const bf16_t one = (bf16_t)1.0f;
   const bf16x8 ones = {one, one, one, one, one, one, one, one};

@@ -1,73 +1,87 @@
-// Attention over the paged cache in true 32-bit: the float path's kernel for prompts and for
-// decoding.  Plain FMA arithmetic (no matrix cores: the float MFMA instructions would want the
-// probabilities moved between lanes, and this path is the check, not the product), but tiled so
-// that keys and values are read once per 32 queries instead of once per query.
+// Attention over the paged cache in true 32-bit: the float path's kernels for prompts and for
+// decoding.  Head sizes: multiples of 16 up to 128 (others take the plain kernel).
 //
-// A work-group of four waves takes 32 consecutive queries of one sequence and one head, and walks
-// the sequence's blocks of 64 keys in order:
-//   * the block's keys [64][hd] and values [16][hd][4] are copied into LDS as they lie in the
-//     cache (the next block's are already in flight into registers meanwhile);
-//   * scores: lane = key, wave = eight of the queries; a lane reads its key row 16 bytes at a
-//     time (rows padded by 16 bytes: conflict-free) against the queries' rows (broadcast reads);
-//   * online softmax: a query's 64 scores lie across the lanes of one wave, so maximum and sum
-//     are wave reductions in registers; excluded scores are replaced by -inf, a block that a
-//     query sees nothing of changes nothing for it (exactly), and a query that sees no key at
-//     all gets zeros;
-//   * values: lane = channel (two channels per lane beyond 64), the same eight queries; the
-//     cache's value layout (four positions interleaved per channel) makes a lane's read of four
-//     keys one 16-byte LDS read, against the probabilities (broadcast reads).
+// Prompts and chunks run on the matrix units.  v_mfma_f32_16x16x4_f32 multiplies and adds in full
+// 32-bit (no reduced-precision mode exists in it), and the arrangement of the bfloat16 kernels
+// needs no probabilities moved between lanes here either:
+//   scores^T [key][query] = K . Q^T: keys are the "A" rows, queries the "B" columns, and a lane
+//       (column lane % 16, group g = lane / 16) ends up with keys 4 g + r (r = 0..3) of each tile
+//       of 16 keys for ONE query.  A 16-byte read gives a lane four channels; the four
+//       instructions that take them multiply channel 16 c + 4 g + r in K index g of step r, the
+//       same for both operands, so every channel is taken exactly once.
+//   out^T [channel][query] = V^T . P^T: in step r of a tile of 16 keys the K index g stands for
+//       key 4 g + r, so the "B" operand is the lane's OWN probability r, and the "A" operand
+//       (channel lane % 16 of a block of 16 channels, key 4 g + r) is element r of ONE 16-byte
+//       read, because the cache keeps four consecutive positions of a channel together.
+// A work-group of four waves takes 64 consecutive queries of one sequence and head, 16 per wave,
+// and walks the sequence's blocks of 64 keys up to its last query:
+//   * the block's keys [64][hd] (rows 16 bytes apart in the banks) and values [16][hd][4] are
+//     copied into LDS as they lie in the cache, once per work-group (the next block's are already
+//     in flight into registers meanwhile);
+//   * the softmax is per query and per block of 64 keys: maximum, rescaling and sum are taken
+//     anew at every block, nothing lags; excluded scores are replaced by -inf, a block that a
+//     query sees nothing of changes nothing for it (exactly), and a query that sees no key at all
+//     gets zeros;
+//   * values of positions behind the tile's last query (which may hold anything, NaN included,
+//     and 0 * NaN is NaN) are replaced by zero once, when the block is staged.
 // A query's result depends on its own keys and on the block boundaries only, which lie at
 // multiples of 64 positions whatever the step: the same arithmetic in the same order whatever
 // else the step holds.  (Steps of one token per sequence have a kernel of their own, below.)
-//
-// Head sizes: multiples of 16 up to 128.
-
-#include <type_traits>
-
+// Measured at 25 heads of 64, 2 x 1,024 tokens: 87 us a layer, 77 TFLOP/s, half of the float
+// MFMA peak; the FMA kernel this replaced (lane = key for the scores, lane = channel for the
+// values, probabilities through LDS) took 445 us.
 #include "host.h"
 #include "attention.h"
 #include "calls.h"
 
-#define F32_QUERIES 32
-#define F32_WAVE_QUERIES 8
+#define F32M_QUERIES 64
 
-template <int CPT>   // channels per lane: 1 (head sizes up to 64) or 2 (up to 128)
+template <int HD>
 __global__ void __launch_bounds__(256)
-attention_f32_kernel(AttnArgs a) {
-  constexpr int MAX_HD = 64 * CPT;
-  constexpr int LOADS = BT_KV_BLOCK * MAX_HD / 4 / 256;      // 16-byte pieces of a block per thread
-  extern __shared__ __attribute__((aligned(16))) float lds[];  // sized for MAX_HD (lds_bytes below)
-  float* qs = lds;                                             // [32][hd]
-  float* ks = qs + F32_QUERIES * MAX_HD;                       // [64][hd + 4]
-  float* vs = ks + BT_KV_BLOCK * (MAX_HD + 4);                 // [16][hd][4], as in the cache
-  float* ps = vs + BT_KV_BLOCK * MAX_HD;                       // [32][64]
+attention_f32_mfma_kernel(AttnArgs a) {
+  constexpr int KS = HD / 16;                                // 16-byte reads of a row per lane; blocks of 16 channels
+  constexpr int LOADS = BT_KV_BLOCK * HD / 4 / 256;          // 16-byte pieces of a block per thread
+  constexpr int K_ROW = HD + 4;                              // floats: rows 16 bytes apart in the banks
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* ks = lds;                                           // [64][HD + 4]
+  float* vs = ks + BT_KV_BLOCK * K_ROW;                      // [16][HD][4], as in the cache
 
-  const int hd = a.kv.head_dim;
-  const int q_tiles = (a.max_count + F32_QUERIES - 1) / F32_QUERIES;
-  const int seq = blockIdx.x / q_tiles, tile = blockIdx.x % q_tiles;
-  const int head = blockIdx.y, kv_head = head / (a.q_heads / a.kv.kv_heads);
+  // The tiles are numbered latest first over the whole grid: a tile's walk is as long as its
+  // position, nearly all work-groups are resident at once, and a compute unit is given every
+  // 256th of them, so that each gets long and short ones.  (Numbered sequence by sequence, a
+  // unit drew tiles of one length: 152 -> 87 us a layer at 2 x 1,024 tokens of 25 heads.)
+  const int q_tiles = (a.max_count + F32M_QUERIES - 1) / F32M_QUERIES;
+  const int units = a.n_seqs * a.q_heads;
+  const int tile = q_tiles - 1 - blockIdx.x / units, unit = blockIdx.x % units;
+  const int seq = unit / a.q_heads, head = unit % a.q_heads, kv_head = head / (a.q_heads / a.kv.kv_heads);
   const int off = a.seq_off[seq], count = a.seq_off[seq + 1] - off, start = a.seq_start[seq];
-  const int q0 = tile * F32_QUERIES;
-  if (q0 >= count) return;                                    // the whole work-group: no barrier is left waiting
+  const int q0 = tile * F32M_QUERIES;
+  if (q0 >= count) return;                                   // the whole work-group: no barrier is left waiting
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n_queries = count - q0 < F32_QUERIES ? count - q0 : F32_QUERIES;
+  const int i16 = lane & 15, g = lane >> 4;
+  const int n_queries = count - q0 < F32M_QUERIES ? count - q0 : F32M_QUERIES;
   const int first_pos = start + q0, last_pos = first_pos + n_queries - 1;
   const int lo_pos = (a.window > 0 && first_pos - a.window + 1 > 0) ? first_pos - a.window + 1 : 0;
   const int first_block = lo_pos / BT_KV_BLOCK, last_block = last_pos / BT_KV_BLOCK;
-  const bool wave_active = wave * F32_WAVE_QUERIES < n_queries;   // else its eight queries do not exist
+  const bool wave_active = wave * 16 < n_queries;
+  // what the wave's queries can see at all: positions wave_lo .. wave_hi
+  const int wave_first = first_pos + wave * 16;
+  const int wave_hi = wave_first + 15 < last_pos ? wave_first + 15 : last_pos;
+  const int wave_lo = (a.window > 0 && wave_first - a.window + 1 > 0) ? wave_first - a.window + 1 : 0;
+  const int mine = wave * 16 + i16;                          // the lane's query within the tile
+  const bool exists = wave_active && mine < n_queries;
+  const int qpos = exists ? first_pos + mine : -1;           // (a column without a query sees no key and is never stored)
 
-  // the queries' rows; rows that do not exist stay zero and are never stored
   const float* q = static_cast<const float*>(a.q);
-  for (int i = tid; i < F32_QUERIES * (hd / 4); i += 256) {
-    int row = i / (hd / 4), c4 = i % (hd / 4);
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (row < n_queries) v = *reinterpret_cast<const float4*>(q + (int64_t)(off + q0 + row) * a.ldq + head * hd + c4 * 4);
-    *reinterpret_cast<float4*>(qs + row * hd + c4 * 4) = v;
+  floatx4 qreg[KS];
+  {
+    const float* row = q + (int64_t)(off + q0 + (exists ? mine : 0)) * a.ldq + head * HD;
+#pragma unroll
+    for (int c = 0; c < KS; ++c) qreg[c] = *reinterpret_cast<const floatx4*>(row + 16 * c + 4 * g);
   }
 
   const float* keys = static_cast<const float*>(a.kv.keys);
   const float* values = static_cast<const float*>(a.kv.values);
-  const int pieces = BT_KV_BLOCK * hd / 4;                   // 16-byte pieces of a block's keys (and of its values)
   floatx4 kreg[LOADS], vreg[LOADS];
   auto fetch = [&](int block) __attribute__((always_inline)) {
     int physical = a.kv.blocks[(int64_t)seq * a.kv.max_blocks + block];
@@ -75,143 +89,127 @@ attention_f32_kernel(AttnArgs a) {
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
       int piece = tid + 256 * j;
-      int at = piece < pieces ? piece : 0;                    // pieces beyond a smaller head size: read the first, keep none
-      kreg[j] = *reinterpret_cast<const floatx4*>(keys + base + (int64_t)at * 4);
-      vreg[j] = *reinterpret_cast<const floatx4*>(values + base + (int64_t)at * 4);
+      kreg[j] = *reinterpret_cast<const floatx4*>(keys + base + (int64_t)piece * 4);
+      vreg[j] = *reinterpret_cast<const floatx4*>(values + base + (int64_t)piece * 4);
     }
   };
-  // Positions behind the tile's last query hold no token of this step and may hold anything, NaN
-  // included (a block that another sequence used before), and 0 * NaN is NaN: their values are
-  // replaced by zero here, once per block and only in the sequence's last block, so that the
-  // multiplications below need no test of their own (a select beside every FMA cost the value
-  // phase half its time).  Everything at or before the last query is a token of this sequence.
+  // (values of positions behind the tile's last query become zero here, once per block and only
+  // in the sequence's last block, so that the multiplications need no test of their own)
   auto stage = [&](int block) __attribute__((always_inline)) {
-    const int beyond = last_pos - block * BT_KV_BLOCK;        // positions of the block above this hold no token
+    const int beyond = last_pos - block * BT_KV_BLOCK;
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
       int piece = tid + 256 * j;
-      if (piece < pieces) {
-        int row = piece / (hd / 4), c4 = piece % (hd / 4);
-        *reinterpret_cast<floatx4*>(ks + row * (hd + 4) + c4 * 4) = kreg[j];
-        floatx4 v = vreg[j];
-        if (beyond < BT_KV_BLOCK - 1) {                       // (the same for the whole work-group)
-          int first = (piece / hd) * 4;                       // the piece holds positions first .. first + 3 of one channel
+      int row = piece / (HD / 4), c4 = piece % (HD / 4);
+      *reinterpret_cast<floatx4*>(ks + row * K_ROW + c4 * 4) = kreg[j];
+      floatx4 v = vreg[j];
+      if (beyond < BT_KV_BLOCK - 1) {                        // (the same for the whole work-group)
+        int first = (piece / HD) * 4;                        // the piece holds positions first .. first + 3 of one channel
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (first + r > beyond) v[r] = 0.f;
-        }
-        *reinterpret_cast<floatx4*>(vs + piece * 4) = v;
+        for (int r = 0; r < 4; ++r)
+          if (first + r > beyond) v[r] = 0.f;
       }
+      *reinterpret_cast<floatx4*>(vs + piece * 4) = v;
     }
   };
 
-  float run_max[F32_WAVE_QUERIES], run_sum[F32_WAVE_QUERIES], acc[F32_WAVE_QUERIES][CPT];
+  const float c2 = a.scale * 1.4426950408889634f;            // scores to powers of two
+  float run_max = -INFINITY, run_sum = 0.f;                  // run_sum: the lane's share; the four lanes of a query meet at the end
+  floatx4 o[KS];
 #pragma unroll
-  for (int i = 0; i < F32_WAVE_QUERIES; ++i) {
-    run_max[i] = -INFINITY;
-    run_sum[i] = 0.f;
-#pragma unroll
-    for (int j = 0; j < CPT; ++j) acc[i][j] = 0.f;
-  }
-  const int my_q = wave * F32_WAVE_QUERIES;                   // first of the wave's queries in the tile
-  // how many of the wave's eight queries exist (one, when decoding): the same in all lanes, so
-  // the tests on it below are scalar branches around work nobody needs
-  const int nq = __builtin_amdgcn_readfirstlane(n_queries - my_q < F32_WAVE_QUERIES ? n_queries - my_q : F32_WAVE_QUERIES);
+  for (int dt = 0; dt < KS; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   fetch(first_block);
   for (int block = first_block; block <= last_block; ++block) {
-    __syncthreads();                                          // the previous block's LDS is no longer read
+    __syncthreads();                                         // the previous block's LDS is no longer read
     stage(block);
-    if (block < last_block) fetch(block + 1);                 // in flight while this block is worked on
+    if (block < last_block) fetch(block + 1);                // in flight while this block is worked on
     __syncthreads();
-    float rescale[F32_WAVE_QUERIES];
-    // ALL: the wave's eight queries all exist (a prompt's interior): no tests in the loops
-    auto score_phase = [&](auto all) __attribute__((always_inline)) {
-      constexpr bool ALL = decltype(all)::value;
-      // scores of key `lane` of the block for the wave's eight queries
-      float s[F32_WAVE_QUERIES];
+    const int kb = block * BT_KV_BLOCK;
+    if (!wave_active || kb > wave_hi || kb + BT_KV_BLOCK <= wave_lo) continue;   // (the same for the whole wave)
+    // Operands are asked for a step before they are multiplied (two sets of registers, named at
+    // compile time), and the four tiles' sums (then the blocks of output channels) take turns, so
+    // that neither an LDS read nor a matrix instruction waits for the one before it.
+    floatx4 s[4];
 #pragma unroll
-      for (int i = 0; i < F32_WAVE_QUERIES; ++i) s[i] = 0.f;
-      const float* krow = ks + lane * (hd + 4);
-      for (int c = 0; c < hd; c += 4) {
-        float4 kv4 = *reinterpret_cast<const float4*>(krow + c);
+    for (int t = 0; t < 4; ++t) s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const float* krow = ks + i16 * K_ROW + 4 * g;
+    floatx4 k4[2][4];
 #pragma unroll
-        for (int i = 0; i < F32_WAVE_QUERIES; ++i) {
-          if (!ALL && i >= nq) continue;
-          float4 q4 = *reinterpret_cast<const float4*>(qs + (my_q + i) * hd + c);
-          s[i] = fmaf(q4.x, kv4.x, s[i]);
-          s[i] = fmaf(q4.y, kv4.y, s[i]);
-          s[i] = fmaf(q4.z, kv4.z, s[i]);
-          s[i] = fmaf(q4.w, kv4.w, s[i]);
-        }
+    for (int t = 0; t < 4; ++t) k4[0][t] = *reinterpret_cast<const floatx4*>(krow + 16 * t * K_ROW);
+#pragma unroll
+    for (int c = 0; c < KS; ++c) {
+      if (c + 1 < KS) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) k4[(c + 1) & 1][t] = *reinterpret_cast<const floatx4*>(krow + 16 * t * K_ROW + 16 * (c + 1));
       }
-      const int key_pos = block * BT_KV_BLOCK + lane;
 #pragma unroll
-      for (int i = 0; i < F32_WAVE_QUERIES; ++i) {
-        rescale[i] = 1.f;
-        if (!ALL && i >= nq) continue;
-        int pos = first_pos + my_q + i;
-        bool seen = key_pos <= pos && (a.window <= 0 || key_pos > pos - a.window);
-        float score = seen ? s[i] * a.scale : -INFINITY;
-        float new_max = fmaxf(run_max[i], wave_max(score));
-        // nothing seen so far, this block included: everything stays at its start
-        float p = new_max == -INFINITY ? 0.f : expf(score - new_max);
-        rescale[i] = new_max == -INFINITY ? 1.f : expf(run_max[i] - new_max);    // exp(-inf) = 0 at the first block seen
-        run_sum[i] = fmaf(run_sum[i], rescale[i], wave_sum(p));     // spelled out: the same in both forms
-        run_max[i] = new_max;
-        ps[(my_q + i) * BT_KV_BLOCK + lane] = p;
-      }
-    };
-    if (wave_active) {
-      if (nq == F32_WAVE_QUERIES) score_phase(std::true_type{}); else score_phase(std::false_type{});
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) s[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(k4[c & 1][t][r], qreg[c][r], s[t], 0, 0, 0);
     }
-    __syncthreads();                                          // the probabilities are in LDS
-    auto value_phase = [&](auto all) __attribute__((always_inline)) {
-      constexpr bool ALL = decltype(all)::value;
+    const float* vcol = vs + (g * HD + i16) * 4;
+    floatx4 v4[2][KS];
 #pragma unroll
-      for (int i = 0; i < F32_WAVE_QUERIES; ++i)
+    for (int dt = 0; dt < KS; ++dt) v4[0][dt] = *reinterpret_cast<const floatx4*>(vcol + 64 * dt);
+    // a block that every query of the wave sees whole needs no comparisons
+    const bool whole = kb + BT_KV_BLOCK - 1 <= wave_first && (a.window <= 0 || kb > wave_hi - a.window);
+    if (!whole) {
 #pragma unroll
-        for (int j = 0; j < CPT; ++j) acc[i][j] *= rescale[i];
-      // values: channel lane (+ 64) of four keys at a time.  Unrolled by two: measured at 2 x 1,024
-      // tokens of 25 heads of 64, 461 / 445 / 546 us a layer unrolled by 1 / 2 / 4 (whole, the
-      // compiler hoists every read above the arithmetic and spills: 1,900 us)
-#pragma unroll 2
-      for (int k4 = 0; k4 < BT_KV_BLOCK / 4; ++k4) {
-        float4 v4[CPT];
+      for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int j = 0; j < CPT; ++j) {
-          int channel = lane + 64 * j;
-          v4[j] = channel < hd ? *reinterpret_cast<const float4*>(vs + (k4 * hd + channel) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int r = 0; r < 4; ++r) {
+          const int key_pos = kb + 16 * t + 4 * g + r;
+          const bool seen = key_pos <= qpos && (a.window <= 0 || key_pos > qpos - a.window);
+          s[t][r] = seen ? s[t][r] : -INFINITY;
         }
+    }
+    float top = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < F32_WAVE_QUERIES; ++i) {
-          if (!ALL && i >= nq) continue;
-          float4 p4 = *reinterpret_cast<const float4*>(ps + (my_q + i) * BT_KV_BLOCK + k4 * 4);
+    for (int t = 0; t < 4; ++t) top = fmaxf(top, fmaxf(fmaxf(s[t][0], s[t][1]), fmaxf(s[t][2], s[t][3])));
+    top = fmaxf(top, __shfl_xor(top, 16, 64));
+    top = fmaxf(top, __shfl_xor(top, 32, 64));
+    const float new_max = fmaxf(run_max, top * c2);          // in powers of two
+    // nothing seen so far, this block included: everything stays at its start
+    const float rescale = new_max == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(run_max - new_max);   // 2^-inf = 0 at the first block seen
+    const float m_use = new_max == -INFINITY ? 0.f : new_max;
+    float block_sum = 0.f;
 #pragma unroll
-          for (int j = 0; j < CPT; ++j) {
-            // (values of positions that hold no token were zeroed when the block was staged)
-            acc[i][j] = fmaf(p4.x, v4[j].x, acc[i][j]);
-            acc[i][j] = fmaf(p4.y, v4[j].y, acc[i][j]);
-            acc[i][j] = fmaf(p4.z, v4[j].z, acc[i][j]);
-            acc[i][j] = fmaf(p4.w, v4[j].w, acc[i][j]);
-          }
-        }
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[t][r] = __builtin_amdgcn_exp2f(fmaf(s[t][r], c2, -m_use));
+        block_sum += s[t][r];
       }
-    };
-    if (wave_active) {
-      if (nq == F32_WAVE_QUERIES) value_phase(std::true_type{}); else value_phase(std::false_type{});
+    run_sum = fmaf(run_sum, rescale, block_sum);
+    run_max = new_max;
+#pragma unroll
+    for (int dt = 0; dt < KS; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] *= rescale;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (t + 1 < 4) {
+#pragma unroll
+        for (int dt = 0; dt < KS; ++dt) v4[(t + 1) & 1][dt] = *reinterpret_cast<const floatx4*>(vcol + 16 * (t + 1) * HD + 64 * dt);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int dt = 0; dt < KS; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(v4[t & 1][dt][r], s[t][r], o[dt], 0, 0, 0);
     }
   }
-  if (wave_active) {
-    float* out = static_cast<float*>(a.out);
+  float total = run_sum;
+  total += __shfl_xor(total, 16, 64);
+  total += __shfl_xor(total, 32, 64);
+  if (exists) {
+    float* out = static_cast<float*>(a.out) + (int64_t)(off + q0 + mine) * a.ldo + head * HD;
 #pragma unroll
-    for (int i = 0; i < F32_WAVE_QUERIES; ++i) {
+    for (int dt = 0; dt < KS; ++dt) {
+      floatx4 r4;
 #pragma unroll
-      for (int j = 0; j < CPT; ++j) {
-        int channel = lane + 64 * j;
-        if (my_q + i < n_queries && channel < hd)
-          out[(int64_t)(off + q0 + my_q + i) * a.ldo + head * hd + channel] = run_sum[i] > 0.f ? acc[i][j] / run_sum[i] : 0.f;
-      }
+      for (int r = 0; r < 4; ++r) r4[r] = total > 0.f ? o[dt][r] / total : 0.f;
+      *reinterpret_cast<floatx4*>(out + 16 * dt + 4 * g) = r4;
     }
   }
 }
@@ -363,6 +361,25 @@ attention_f32_join_kernel(AttnArgs a) {
   }
 }
 
+template <int HD>
+static int launch_prompt(hipStream_t stream, const AttnArgs& a) {
+  const int q_tiles = (a.max_count + F32M_QUERIES - 1) / F32M_QUERIES;
+  const size_t lds = sizeof(float) * (size_t)(BT_KV_BLOCK * (HD + 4) + BT_KV_BLOCK * HD);
+  if (lds > 64 * 1024) {                        // beyond what a kernel gets without asking
+    static bool raised = false;
+    if (!raised) {
+      hipError_t err = hipFuncSetAttribute((const void*)attention_f32_mfma_kernel<HD>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (err != hipSuccess) BT_REFUSE("attention_f32: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));
+      raised = true;
+    }
+  }
+  const int64_t groups = (int64_t)a.n_seqs * a.q_heads * q_tiles;
+  if (groups > 0x7fffffff) BT_REFUSE("attention_f32: %lld work-groups are too many", (long long)groups);
+  hipLaunchKernelGGL(attention_f32_mfma_kernel<HD>, dim3((unsigned)groups), dim3(256), lds, stream, a);
+  return bt_check_launch("attention_f32");
+}
+
 BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
   if (args->out_rows != 0) BT_REFUSE("attention_f32: a chunk-major output is written by the bfloat16 decode kernel only");
   const AttnArgs& a = *args;
@@ -394,25 +411,18 @@ BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
     }
     return bt_check_launch("attention_f32");
   }
-  const int q_tiles = (a.max_count + F32_QUERIES - 1) / F32_QUERIES;
-  dim3 grid(a.n_seqs * q_tiles, a.q_heads), block(256);
-  auto lds_bytes = [](int max_hd) {
-    return sizeof(float) * (size_t)(F32_QUERIES * max_hd + BT_KV_BLOCK * (max_hd + 4) + BT_KV_BLOCK * max_hd +
-                                    F32_QUERIES * BT_KV_BLOCK);
-  };
-  if (hd <= 64) {
-    hipLaunchKernelGGL(attention_f32_kernel<1>, grid, block, lds_bytes(64), (hipStream_t)stream, a);
-  } else {
-    static bool raised = false;                 // 90 KB: beyond what a kernel gets without asking
-    if (!raised) {
-      hipError_t err = hipFuncSetAttribute((const void*)attention_f32_kernel<2>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(128));
-      if (err != hipSuccess) BT_REFUSE("attention_f32: cannot get %zu bytes of LDS: %s", lds_bytes(128), hipGetErrorString(err));
-      raised = true;
-    }
-    hipLaunchKernelGGL(attention_f32_kernel<2>, grid, block, lds_bytes(128), (hipStream_t)stream, a);
+  if (a.ldo % 4 != 0 || ((uintptr_t)a.out & 15))
+    BT_REFUSE("attention_f32: output rows are written 16 bytes at a time (row pitch %lld)", (long long)a.ldo);
+  switch (hd) {
+    case 16: return launch_prompt<16>((hipStream_t)stream, a);
+    case 32: return launch_prompt<32>((hipStream_t)stream, a);
+    case 48: return launch_prompt<48>((hipStream_t)stream, a);
+    case 64: return launch_prompt<64>((hipStream_t)stream, a);
+    case 80: return launch_prompt<80>((hipStream_t)stream, a);
+    case 96: return launch_prompt<96>((hipStream_t)stream, a);
+    case 112: return launch_prompt<112>((hipStream_t)stream, a);
+    default: return launch_prompt<128>((hipStream_t)stream, a);
   }
-  return bt_check_launch("attention_f32");
 }
 
 // The same entry points with their arguments as one structure (calls.h), for launch lists.

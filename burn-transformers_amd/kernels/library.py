@@ -647,7 +647,8 @@ def attention(args, dtype, decode, impl="auto"):
         if code == BFLOAT16:
             impl = "mfma"
         else:
-            impl = "tiled" if args.kv.head_dim <= 128 and args.kv.head_dim % 16 == 0 and args.ldq % 4 == 0 else "plain"
+            impl = "tiled" if args.kv.head_dim <= 128 and args.kv.head_dim % 16 == 0 and args.ldq % 4 == 0 \
+                and (decode or args.ldo % 4 == 0) else "plain"
     call = AttentionCall(dtype=code, args=args)
     if impl == "plain":
         _launch(_module("core"), "bt_attention_plain_call", call)

@@ -18,9 +18,9 @@
 //                      32 queries (two MFMA column tiles, which share every key and value load)
 //                      and walks the keys up to its last query's position.  (Four column tiles
 //                      per wave were measured and were slower: they leave one wave per SIMD.)
-//                      Heads of 64 without a window: eight waves, keys and values through LDS,
-//                      each block of keys taken by one of two sets of waves
-//                      (attention_prefill_split_kernel).
+//                      Heads of 64 without a window: eight waves, keys and values through LDS
+//                      (brought there by four waves that do nothing else), each block of keys
+//                      taken by one of two sets of waves (attention_prefill_split_kernel).
 //   attention_decode   one token per sequence: one work-group per (key/value head, sequence)
 //                      and run of keys; the query heads sharing that head are the MFMA columns;
 //                      eight waves split the keys and meet in LDS; the runs of a long context
@@ -487,18 +487,30 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 // the rate and 36 matrix instructions per block); the loads cost 80 us, the writes 28, the
 // barrier 39.  Keeping three turns in LDS, so that operands are read a turn ahead and nobody
 // waits at the barrier, and reading the block table a turn ahead were both tried and gained
-// nothing: the cost of those parts is their instructions, not their waiting.
+// nothing: the cost of those parts is their instructions, not their waiting.  So the loads and
+// the writes were given to waves of their own (below): 8,192 tokens 448 -> 349 us (616 TFLOP/s),
+// 2,048 tokens 38.9 -> 34.6 us, 2 x 1,024 tokens 24.7 -> 23.7 us.
 #define SPLIT_TURN (2 * SHARED_STAGE)
 #define SPLIT_LDS_BYTES (2 * SPLIT_TURN)
 
-__global__ void __launch_bounds__(2 * PREFILL_WAVES * 64)
+// Four more waves do nothing but bring the blocks in (SPLIT_PRODUCERS): they ask memory for the
+// turn after next, write the next turn's blocks from their registers into the LDS stage that
+// everyone has left, and meet the others at the turn's barrier.  The time of the eight waves
+// that multiply is their own instruction streams, so what they do not have to issue they do not
+// pay for, and the bringers' streams run beside them on the same SIMDs (160 registers: three
+// waves a SIMD).
+#define SPLIT_PRODUCERS 4
+#define SPLIT_THREADS ((2 * PREFILL_WAVES + SPLIT_PRODUCERS) * 64)
+
+__global__ void __launch_bounds__(SPLIT_THREADS)
 attention_prefill_split_kernel(AttnArgs a) {
-  constexpr int THREADS = 2 * PREFILL_WAVES * 64;
-  static_assert(THREADS == 512, "one 16-byte piece of a block's keys and one of its values per thread");
+  static_assert(2 * PREFILL_WAVES * 64 == 512 && SPLIT_PRODUCERS * 64 == 256,
+                "two 16-byte pieces of a block's keys and two of its values per bringing thread");
   typedef __attribute__((__vector_size__(4 * sizeof(int)))) int int4v;
   extern __shared__ __attribute__((aligned(16))) unsigned char split_lds[];   // [2 turns][2 blocks][SHARED_STAGE]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool brings = wave8 >= 2 * PREFILL_WAVES;           // (the same for a whole wave: a scalar branch)
   const int set = wave8 / PREFILL_WAVES, wave = wave8 % PREFILL_WAVES;
   const int i16 = lane & 15, g = lane >> 4;
   // work-groups that read the same keys and values lie on one XCD (as in attention_prefill_kernel);
@@ -519,8 +531,63 @@ attention_prefill_split_kernel(AttnArgs a) {
   const int reach = (q_tile + 1) * PREFILL_QUERIES < count ? (q_tile + 1) * PREFILL_QUERIES : count;
   const int n_blocks = (start + reach + BT_KV_BLOCK - 1) / BT_KV_BLOCK;
   const int n_turns = (n_blocks + 1) / 2;
+  // Every wave meets the others at the same barriers: one when the first turn is in place, one at
+  // the end of every turn, one before the second set's results are read.
+
+  if (brings) {
+    const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
+    const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
+    typedef __attribute__((__vector_size__(2 * sizeof(int)))) int int2v;
+    const int mine = tid - 2 * PREFILL_WAVES * 64;           // 0 .. 255: pieces mine and mine + 256 of each plane
+    int4v kreg[2][2], vreg[2][2];
+    auto fetch = [&](int turn) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        int block_index = 2 * turn + b;
+        if (block_index >= n_blocks) block_index = n_blocks - 1;     // (read again, never multiplied)
+        int64_t plane = tile_plane(a, seq, kv_head, block_index * BT_KV_BLOCK);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          kreg[b][h] = *reinterpret_cast<const int4v*>(keys + plane + (mine + 256 * h) * 8);
+          vreg[b][h] = *reinterpret_cast<const int4v*>(values + plane + (mine + 256 * h) * 8);
+        }
+      }
+    };
+    auto stash = [&](unsigned char* turn_base) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        unsigned char* stage = turn_base + b * SHARED_STAGE;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int piece = mine + 256 * h;
+          const int row = piece >> 3, chunk = piece & 7;
+          *reinterpret_cast<int4v*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4)) = kreg[b][h];
+          // a piece of the values: positions 4 * four .. + 3 of channels 2 * pair and 2 * pair + 1,
+          // eight bytes each, to the halves of two neighbouring operands
+          const int four = piece >> 5, pair = piece & 31;
+          unsigned char* place = stage + SHARED_K_BYTES + (((four >> 3) * 4 + (four & 3)) * 64 + 2 * pair) * 16 +
+                                 ((four >> 2) & 1) * 8;
+          *reinterpret_cast<int2v*>(place) = int2v{vreg[b][h][0], vreg[b][h][1]};
+          *reinterpret_cast<int2v*>(place + 16) = int2v{vreg[b][h][2], vreg[b][h][3]};
+        }
+      }
+    };
+    fetch(0);
+    stash(split_lds);
+    if (n_turns > 1) fetch(1);
+    __syncthreads();                                         // the first turn is in place
+    for (int t = 0; t < n_turns; ++t) {
+      // the place of turn t + 1 was read in turn t - 1, which everyone has left
+      if (t + 1 < n_turns) stash(split_lds + ((t + 1) & 1) * SPLIT_TURN);
+      if (t + 2 < n_turns) fetch(t + 2);
+      __syncthreads();                                       // the end of turn t
+    }
+    __syncthreads();                                         // (before the second set's results are read)
+    return;
+  }
+
   const int q0 = q_tile * PREFILL_QUERIES + wave * PREFILL_QUERIES_PER_WAVE;
-  const bool active = q0 < count;                           // (a wave without queries still moves its share of every block)
+  const bool active = q0 < count;
   const bf16_t* Q = static_cast<const bf16_t*>(a.q);
 
   int qpos[PREFILL_NQ], tok[PREFILL_NQ];
@@ -546,39 +613,9 @@ attention_prefill_split_kernel(AttnArgs a) {
   const int valid_end = start + count;
   const float c = a.scale * LOG2_E;
   const int whole_until = start + q0 + 1;       // blocks ending here or before are seen whole
-  const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
-  const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
 
-  typedef __attribute__((__vector_size__(2 * sizeof(int)))) int int2v;
-  int4v kreg[2], vreg[2];
-  auto fetch = [&](int turn) {
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      int block_index = 2 * turn + b;
-      if (block_index >= n_blocks) block_index = n_blocks - 1;     // (read again, never multiplied)
-      int64_t plane = tile_plane(a, seq, kv_head, block_index * BT_KV_BLOCK);
-      kreg[b] = *reinterpret_cast<const int4v*>(keys + plane + tid * 8);
-      // the thread's values: one channel, the two groups of four positions that one operand holds
-      const bf16_t* mine = values + plane + ((tid >> 8) * 8 + ((tid >> 6) & 3)) * (4 * HD) + (tid & 63) * 4;
-      const int2v low = *reinterpret_cast<const int2v*>(mine), high = *reinterpret_cast<const int2v*>(mine + 16 * HD);
-      vreg[b] = int4v{low[0], low[1], high[0], high[1]};
-    }
-  };
-  auto stash = [&](unsigned char* turn_base) {
-    const int row = tid >> 3, chunk = tid & 7;
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      unsigned char* stage = turn_base + b * SHARED_STAGE;
-      *reinterpret_cast<int4v*>(stage + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4)) = kreg[b];
-      *reinterpret_cast<int4v*>(stage + SHARED_K_BYTES + tid * 16) = vreg[b];   // ((4 h + g) * 64 + channel) * 16
-    }
-  };
-  fetch(0);
-  stash(split_lds);
-  __syncthreads();
+  __syncthreads();                              // the first turn is in place
   for (int t = 0; t < n_turns; ++t) {
-    const bool more = t + 1 < n_turns;
-    if (more) fetch(t + 1);
     const int block_index = 2 * t + set;
     const int kb = block_index * BT_KV_BLOCK;
     if (block_index < n_blocks && kb < hi) {
@@ -599,7 +636,6 @@ attention_prefill_split_kernel(AttnArgs a) {
                                                              ((4 * half + g) * 64 + dt * 16 + i16) * 16);
       attend_block<PREFILL_NQ>(blk, kb, valid_end, kb + 64 > whole_until, qpos, c, q, o, m, rows);
     }
-    if (more) stash(split_lds + ((t + 1) & 1) * SPLIT_TURN);
     __syncthreads();   // turn t + 1 is in place, and everyone is done with turn t before it is overwritten
   }
   // The second set's results go to the first, lane to lane: value k of lane `lane` of wave `wave`
@@ -838,7 +874,7 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
     }
     const int64_t split_groups = 8 * units_per_xcd * group * q_tiles;
     if (split_groups > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: %lld work-groups are too many", (long long)split_groups);
-    hipLaunchKernelGGL(attention_prefill_split_kernel, dim3((unsigned)split_groups), dim3(2 * PREFILL_WAVES * 64), SPLIT_LDS_BYTES,
+    hipLaunchKernelGGL(attention_prefill_split_kernel, dim3((unsigned)split_groups), dim3(SPLIT_THREADS), SPLIT_LDS_BYTES,
                        (hipStream_t)stream, *args);
     return bt_check_launch("attention_prefill_bf16");
   }

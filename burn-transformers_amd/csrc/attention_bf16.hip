@@ -461,9 +461,11 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 //           32 h + 4 g + 0..3 and 32 h + 16 + 4 g + 0..3 of its channel: those 16 bytes lie
 //           together at ((4 h + g) * 64 + channel) * 16, so an operand is ONE ds_read_b128 and
 //           the 16 lanes of a group read 256 consecutive bytes.  (The cache keeps four
-//           consecutive positions of a channel together: a thread brings the two groups of four
-//           positions of ONE channel that belong to one operand, eight bytes each, and stores
-//           them as one 16-byte piece, a wave 1,024 consecutive bytes.)
+//           consecutive positions of a channel together, so a 16-byte piece of it, two channels
+//           of one group of four positions, goes to the halves of two neighbouring operands,
+//           eight bytes each.  Those writes collide in the banks, four lanes to a bank; bringing
+//           one channel's two groups instead, eight bytes each, and writing 16 was measured and
+//           was no faster.)
 #define SHARED_K_BYTES (64 * 128)
 #define SHARED_V_BYTES (64 * 128)
 #define SHARED_STAGE (SHARED_K_BYTES + SHARED_V_BYTES)
@@ -478,7 +480,7 @@ __device__ __forceinline__ void attend_block(const BlockOperands& blk, int kb, i
 // every SIMD has two waves at work all the time instead of one for most of it.  The tiles are
 // numbered latest first over the whole grid, so that the short ones fill in behind the long
 // ones.  Measured at 25 heads: 2 x 1,024 tokens 29.3 -> 27.3 us, 2,048 tokens 50.2 -> 43.2 us,
-// 4 chunks of 256 tokens behind 768 28.4 -> 21.8 us.  With the leaner softmax of block_output
+// 4 chunks of 256 tokens behind 768 28.4 -> 21.8 us.  With the leaner softmax of attend_block
 // (maxima per lane, sums from the matrix unit, values in LDS in operand order): 24.5, 38.5 and
 // 20.3 us, and 8,192 tokens of one sequence 503 -> 445 us (480 TFLOP/s).  What the time goes to
 // then, measured by leaving parts out at 8,192 tokens: with no loads from memory, no writes to

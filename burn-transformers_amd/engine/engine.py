@@ -39,6 +39,18 @@ _PINNED_RING = 4
 _MAX_GRAPHS = 48           # graphs kept; the one that was used longest ago goes first
 _MAX_PROGRAMS = 1024       # launch lists kept (a few hundred small structures each)
 _META_WORDS = 1 << 16      # first size of the device buffer of a step's integer tables
+_PROBES = 3                # steps of a shape that are measured before it is captured or left to its list
+
+
+def launch_bound(samples):
+    """From measured steps of one shape, each (seconds the GPU took from the step's first kernel
+    to its last, seconds the host took to walk its launch list): True if the GPU is the limit, so
+    that a graph would gain nothing.  Where the host is the limit the GPU waits for every launch
+    and both times are about equal; where the kernels outlast their launches the GPU's time is the
+    longer one.  The median ratio decides, so one odd sample (a first use, a clock still rising)
+    does not."""
+    ratios = sorted(gpu / max(host, 1e-9) for gpu, host in samples)
+    return ratios[len(ratios) // 2] > 1.1
 
 
 class StepError(ValueError):
@@ -70,8 +82,9 @@ class Engine:
         self._graphs = {}                  # shape -> dict(graph, meta, logits, generation), in order of last use
         self._seen = {}                    # shape -> times it came without a graph
         # shape -> True (its launch list keeps the GPU busy: no graph), False (the host is the limit:
-        # graph), or the measurement under way: (host seconds, start event, end event)
+        # graph), or the measurements under way: [(host seconds of the walk, start event, end event)]
         self._launch_bound = {}
+        self._walk_seconds = None          # host time of the latest walk of a launch list
         self.graphs_declined = 0           # shapes that were measured and left to their launch lists
         self.steps_run = 0
         self.graph_replays = 0
@@ -99,16 +112,26 @@ class Engine:
 
     # --- the step function -----------------------------------------------------------------
     def plan(self, entries, want=None):
-        """Validates a step and lays its tables out on the host.  Changes nothing."""
-        if not entries:
-            raise StepError("a step needs at least one sequence")
+        """Validates a step and lays its tables out on the host.  Changes nothing.
+
+        An entry that brings no token is idle: it runs nothing, writes nothing and keeps its length
+        (the reference's decode rows without a valid token, src/models/llama/model/decode.rs:43-44).
+        ``active`` names the entries that bring tokens, ``idle_rows`` the places in the step's
+        logits that idle entries take (one row of zeros each when the places are not given:
+        decode.rs:730-751)."""
         ledger = self.cache.ledger
-        slots, starts, counts, ids = [], [], [], []
+        slots, starts, counts, ids, active = [], [], [], [], []
         limit = min(self.model.max_positions, self.cache.max_sequence_length)
         vocab = self.model.vocab_size
-        for slot, tokens in entries:
+        if want is not None and len(want) != len(entries):
+            raise StepError("`want` needs one list of places per sequence")
+        seen = set()
+        for index, (slot, tokens) in enumerate(entries):
             if not ledger.live(slot):
                 raise StepError(f"slot {slot} is not open")
+            if slot in seen:
+                raise StepError(f"slot {slot} appears twice in one step")
+            seen.add(slot)
             if type(tokens) is list and len(tokens) == 1 and type(tokens[0]) is int:
                 size, low, high = 1, tokens[0], tokens[0]      # a decode step's entry: no array is made for it
                 ids.append(tokens[0])
@@ -119,7 +142,9 @@ class Engine:
                 tokens = tokens.astype(np.int64).reshape(-1)
                 size = int(tokens.size)
                 if size == 0:
-                    raise StepError(f"slot {slot} brings no token; leave idle sequences out of the step")
+                    if want is not None and len(want[index]):
+                        raise StepError(f"wanted place {want[index][0]} of slot {slot} is outside its 0 tokens")
+                    continue
                 low, high = int(tokens.min()), int(tokens.max())
                 ids.extend(tokens.tolist())
             if low < 0 or high >= vocab:
@@ -129,21 +154,20 @@ class Engine:
             if start + size > limit:
                 raise StepError(f"slot {slot} would reach {start + size} tokens, "
                                 f"the limit is {limit}")
+            active.append(index)
             slots.append(slot)
             starts.append(start)
             counts.append(size)
-        if len(set(slots)) != len(slots):
-            twice = next(slot for slot in slots if slots.count(slot) > 1)
-            raise StepError(f"slot {twice} appears twice in one step")
-        offsets = np.concatenate([[0], np.cumsum(counts)])
+        offsets = np.concatenate([[0], np.cumsum(counts)]) if counts else np.zeros(1, dtype=np.int64)
+        idle_rows = None
         if want is None:
-            wanted = [int(offsets[i + 1] - 1) for i in range(len(entries))]
+            wanted = [int(offsets[i + 1] - 1) for i in range(len(active))]
+            if len(active) != len(entries):         # a row of zeros for every idle entry, where its logits would be
+                idle_rows = [i for i in range(len(entries)) if i not in set(active)]
         else:
-            if len(want) != len(entries):
-                raise StepError("`want` needs one list of places per sequence")
             wanted = []
-            for i, places in enumerate(want):
-                for place in places:
+            for i, index in enumerate(active):
+                for place in want[index]:
                     if not (0 <= place < counts[i]):
                         raise StepError(f"wanted place {place} of slot {slots[i]} is outside its "
                                         f"{counts[i]} tokens")
@@ -154,7 +178,8 @@ class Engine:
         except RuntimeError as error:
             raise StepError(str(error)) from error
         # block rows are read after the reservation, in `step`
-        return dict(slots=slots, starts=starts, counts=counts, ids=ids, wanted=wanted, new_lengths=new_lengths)
+        return dict(slots=slots, starts=starts, counts=counts, ids=ids, wanted=wanted, new_lengths=new_lengths,
+                    active=active, idle_rows=idle_rows, n_entries=len(entries))
 
     def step(self, entries, want=None, device_tokens=None):
         """Runs one step; returns float32 logits [wanted places, vocab] on the GPU, valid until the
@@ -168,9 +193,15 @@ class Engine:
         The ids are not validated (a selection cannot choose outside the vocabulary)."""
         checked = self.plan(entries, want)
         if device_tokens is not None:
-            if max(checked["counts"]) != 1 or device_tokens.numel() != len(entries) or \
+            if len(checked["active"]) != len(entries) or max(checked["counts"], default=0) != 1 or \
+                    device_tokens.numel() != len(entries) or \
                     device_tokens.dtype != torch.int32 or device_tokens.device != self.device:
                 raise StepError("device_tokens: one int32 token on this GPU for each sequence of a step of single tokens")
+        if not checked["active"]:
+            # No entry brings a token: nothing runs and nothing is committed; the logits are exact
+            # zeros of the shape asked for (src/models/llama/model/decode.rs:648-650, 730-751)
+            return torch.zeros((len(checked["idle_rows"] or ()), self.model.vocab_size), dtype=torch.float32,
+                               device=self.device)
         ledger = self.cache.ledger
         for slot, length in checked["new_lengths"].items():
             ledger.reserve(slot, length)
@@ -195,6 +226,10 @@ class Engine:
         for slot, length in checked["new_lengths"].items():
             ledger.commit(slot, length)
         self.steps_run += 1
+        if checked["idle_rows"]:          # rows of zeros where idle entries' logits would be
+            whole = torch.zeros((checked["n_entries"], self.model.vocab_size), dtype=torch.float32, device=self.device)
+            whole[torch.tensor(checked["active"], device=self.device)] = logits
+            return whole
         return logits
 
     # --- running ---------------------------------------------------------------------------
@@ -240,6 +275,8 @@ class Engine:
         if self._programs_generation != self.pool.generation:
             self._programs.clear()
             self._programs_generation = self.pool.generation
+            # (measurements under way were of lists that are gone; decisions taken stay)
+            self._launch_bound = {k: v for k, v in self._launch_bound.items() if isinstance(v, bool)}
         key = (plan.layout.key(), plan.max_count, readout, plan.context_limit if plan.decode else 0)
         held = self._programs.pop(key, None)
         if held is None:
@@ -266,7 +303,9 @@ class Engine:
             return logits
         self._programs[key] = held                        # (again) the most recently used
         self.last_program = held[0]
+        began = time.perf_counter()
         held[0].run()
+        self._walk_seconds = time.perf_counter() - began
         self.program_runs += 1
         return held[1]
 
@@ -298,39 +337,45 @@ class Engine:
         return held["logits"]
 
     def _graph_pays(self, key, plan, readout):
-        """Whether the shape should be captured, found out by measuring its launch list once.
+        """Whether the shape should be captured, found out by measuring its launch list.
 
         A graph removes the host's cost of launching a step's kernels.  That cost is hidden anyway
         where the kernels keep the GPU busy for longer than the host needs to launch them (every
         dependent kernel takes the GPU some microseconds however little it does, and the C++ walk
         launches one in about three): then a graph gains nothing and costs its capture, a stall of
-        the pipeline, and memory.  So the step that would have been captured runs from its list
-        between two events and the host's time for it is taken; when the shape comes next, the
-        GPU's time is read (one wait, shorter than a capture's) and compared.  Returns False when
-        it ran the step itself (the logits are in ``_latest_logits``)."""
+        the pipeline, and memory.  So the steps that would have been captured run from their list
+        between two events while the host's time for the walk alone is taken (not the upload of the
+        step's tables, which may wait for an older copy); after ``_PROBES`` such steps the GPU's
+        times are read (one wait, shorter than a capture's) and ``launch_bound`` decides by the
+        median.  Returns False when it ran the step itself (the logits are in ``_latest_logits``)."""
         probe = self._launch_bound.get(key)
+        if probe is False:
+            return True
         if probe is None:
             if len(self._launch_bound) > 4096:
                 self._launch_bound.clear()
-            if key not in self._programs and self._seen.get(key, 0) < 8:
-                # the shape has no list yet (its first step made a workspace grow): this step would be
-                # launched from Python and say nothing about the list; it records, the next one is measured
-                self._seen[key] = self._seen.get(key, 0) + 1
-                self._latest_logits = self._run_eager(plan, want_logits=readout)
-                return False
+            probe = self._launch_bound[key] = []
+        if key not in self._programs and self._seen.get(key, 0) < 8:
+            # the shape has no list (its first step made a workspace grow, or the lists were dropped
+            # since): this step would be launched from Python and say nothing about the list; it
+            # records, the next one is measured
+            self._seen[key] = self._seen.get(key, 0) + 1
+            self._latest_logits = self._run_eager(plan, want_logits=readout)
+            return False
+        if len(probe) < _PROBES:
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            began = time.perf_counter()
             start.record()
+            self._walk_seconds = None
             self._latest_logits = self._run_eager(plan, want_logits=readout)
             end.record()
-            self._launch_bound[key] = (time.perf_counter() - began, start, end)
+            if self._walk_seconds is not None:        # (None: the step recorded its list anew and says nothing)
+                probe.append((self._walk_seconds, start, end))
             return False
-        if probe is False:
-            return True
-        host_seconds, start, end = probe
-        end.synchronize()
-        gpu_seconds = start.elapsed_time(end) * 1e-3
-        self._launch_bound[key] = gpu_seconds > 1.1 * host_seconds
+        samples = []
+        for host_seconds, start, end in probe:
+            end.synchronize()
+            samples.append((start.elapsed_time(end) * 1e-3, host_seconds))
+        self._launch_bound[key] = launch_bound(samples)
         if self._launch_bound[key]:
             self.graphs_declined += 1
             self._latest_logits = self._run_eager(plan, want_logits=readout)

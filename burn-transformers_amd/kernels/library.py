@@ -197,13 +197,19 @@ def _check(lib, code):
         raise KernelError(lib.bt_last_error().decode())
 
 
-_recorder = [None]      # the Program that kernels are being written into instead of being launched
+class _Recorder(threading.local):
+    """The Program that this thread's kernel calls are being written into, if any: a list records
+    what the thread that opened it issues, and nothing that another thread launches meanwhile."""
+    program = None
+
+
+_recorder = _Recorder()
 
 
 def _launch(lib, name, call):
     """Calls a kernel's structure form now, or, while a launch list is being recorded, keeps the
     pair for later."""
-    program = _recorder[0]
+    program = _recorder.program
     if program is not None:
         program.add(lib, name, call)
         if not program.launch_while_recording:
@@ -268,13 +274,13 @@ class _Recording:
         self.program = program
 
     def __enter__(self):
-        if _recorder[0] is not None:
+        if _recorder.program is not None:
             raise RuntimeError("a launch list is already being recorded")
-        _recorder[0] = self.program
+        _recorder.program = self.program
         return self.program
 
     def __exit__(self, *exc):
-        _recorder[0] = None
+        _recorder.program = None
         return False
 
 

@@ -12,3 +12,4 @@ for path in (ROOT, os.path.dirname(os.path.abspath(__file__))):
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
     config.addinivalue_line("markers", "slow: takes a minute or more (models of a billion parameters)")
+    config.addinivalue_line("markers", "perf: asserts on measured time; not part of the correctness runs (run with -m perf)")

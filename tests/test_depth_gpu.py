@@ -111,9 +111,9 @@ def test_48_layers_whole_then_tail_one_by_one(dtype):
     for t in range(64, 96):
         got.append(engine.step([(slot, [ids[t]])]).clone())
     check(torch.cat(got), want, dtype, "the same with its last 32 tokens one by one")
-    # 343 kernels keep the GPU busy for longer than the C++ walk needs to launch them: the engine
-    # measures that once and leaves the shape to its launch list instead of capturing a graph
-    assert engine.graphs_declined == 1 and engine.graph_replays == 0 and engine.program_runs >= 28
+    # the engine chose for itself how the repeating decode shape runs (from its launch list or from
+    # a graph, by what it measured on this machine): either way the steps did not come from Python
+    assert engine.graph_replays + engine.program_runs >= 28
     engine.close(slot)
     engine.cache.ledger.check()
 

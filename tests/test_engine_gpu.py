@@ -448,6 +448,51 @@ def test_refused_steps_change_nothing():
     engine.cache.ledger.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_idle_entries_run_nothing_commit_nothing_and_read_as_zeros(dtype):
+    """An entry without tokens is a no-op with exact zero logits, and a step of nothing but such
+    entries commits nothing (src/models/llama/model/decode.rs:43-44, 648-650, 730-751; the
+    reference's test is decode_tests.rs:382): lengths, blocks and the steps counted stay, and the
+    entries beside an idle one get the logits they get without it, bit for bit."""
+    from burn_transformers_amd.engine.engine import StepError
+    name = "A"
+    engine = engine_for(name, dtype, graphs=False)
+    first, second, third = prompts_for(name, [20, 9, 70], seed=31)
+    a, b, c = engine.open(), engine.open(), engine.open()
+    engine.step([(a, first[:10]), (b, second[:8]), (c, third[:64])])
+    ledger = engine.cache.ledger
+    before = (list(ledger.lengths), [list(x) for x in ledger.held_blocks[0]], ledger.blocks[0].available(), engine.steps_run)
+    state = lambda: (list(ledger.lengths), [list(x) for x in ledger.held_blocks[0]], ledger.blocks[0].available(), engine.steps_run)
+    vocab = CONFIGS[name][0]["vocab_size"]
+    # nothing at all, and nothing but idle entries, with and without wanted places
+    assert tuple(engine.step([]).shape) == (0, vocab)
+    zeros = engine.step([(a, []), (b, []), (c, [])])
+    assert tuple(zeros.shape) == (3, vocab) and zeros.dtype == torch.float32 and not zeros.any()
+    assert tuple(engine.step([(a, []), (c, [])], want=[[], []]).shape) == (0, vocab)
+    assert state() == before
+    with pytest.raises(StepError, match="outside its 0 tokens"):
+        engine.step([(a, []), (b, [second[8]])], want=[[0], [0]])
+    assert state() == before
+    # an idle entry between two that go on: its row is zeros, theirs are what they are without it
+    mixed = engine.step([(a, [first[10]]), (b, []), (c, third[64:])]).clone()
+    assert not mixed[1].any()
+    assert [engine.length(s) for s in (a, b, c)] == [11, 8, 70]
+    check(mixed[0:1], plain_logits(name, first[:11])[-1:], dtype, "beside an idle entry, decode row")
+    check(mixed[2:3], plain_logits(name, third)[-1:], dtype, "beside an idle entry, prompt row")
+    engine.truncate(a, 10)
+    engine.truncate(c, 64)
+    alone = engine.step([(a, [first[10]]), (c, third[64:])])
+    assert torch.equal(alone[0], mixed[0]) and torch.equal(alone[1], mixed[2])
+    # wanted places given: the idle entry has none, and takes no row
+    some = engine.step([(a, [first[11]]), (b, []), (c, [])], want=[[0], [], []])
+    assert tuple(some.shape) == (1, vocab)
+    check(some, plain_logits(name, first[:12])[-1:], dtype, "explicit places beside idle entries")
+    # the idle sequence goes on afterwards as if nothing had been
+    check(engine.step([(b, [second[8]])]), plain_logits(name, second)[-1:], dtype, "after idling")
+    ledger.check()
+    engine.reset()
+
+
 @pytest.mark.parametrize("graphs", [False, True])
 def test_tokens_that_are_on_the_gpu_already_feed_a_step_from_there(graphs):
     """``device_tokens``: the step reads its tokens from a tensor on the GPU (what a selection has

@@ -3,8 +3,6 @@
 A list is recorded from the same parts that issue kernels one by one, so both ways run the same
 kernels with the same arguments: every result here is compared bit for bit."""
 
-import time
-
 import pytest
 import torch
 
@@ -116,34 +114,20 @@ def test_a_call_that_refuses_names_itself_and_the_step_changes_nothing():
     assert float((logits.cpu().double() - want).abs().max()) <= tolerance("float32", want)
 
 
-def test_host_time_of_a_listed_step_is_a_fraction_of_the_direct_one():
-    """What the list is for: the host's share of a step.  Measured without waiting for the GPU
-    (the calls only queue work): the same steps issued from Python cost several times more."""
-    model = model_for("BW", "bfloat16")
-    ids = prompts_for("BW", [64], seed=85)[0]
-    seconds = {}
-    for programs in (True, False):
-        engine = bt.Engine(model, max_tokens=64 * 4, graphs=False, programs=programs)
-        slot = engine.open()
-        engine.step([(slot, ids)])
-        engine.truncate(slot, 0)
-        torch.cuda.synchronize()
-        started = time.perf_counter()
-        for _ in range(20):
-            engine.step([(slot, ids)])
-            engine.truncate(slot, 0)
-        seconds[programs] = (time.perf_counter() - started) / 20
-        torch.cuda.synchronize()
-    print(f"host time of a 64-token step of a 3-layer model: {seconds[True] * 1e6:.0f} us from a launch list, "
-          f"{seconds[False] * 1e6:.0f} us call by call")
-    assert seconds[True] < 0.7 * seconds[False]
+@pytest.mark.parametrize("gpu_is_the_limit", [False, True])
+def test_a_measured_shape_is_captured_or_left_to_its_list(gpu_is_the_limit, monkeypatch):
+    """The engine's own choice (graphs=True) with the verdict of the measurement given: a repeating
+    shape runs from Python once (its list is recorded), from its list while it is measured, and
+    then from a graph if the host was found to be the limit, else from its list for good.  The
+    logits are the plain implementation's on either path."""
+    from burn_transformers_amd.engine import engine as engine_module
+    seen = []
 
+    def verdict(samples):
+        seen.append(samples)
+        return gpu_is_the_limit
 
-def test_a_small_model_whose_launches_outlast_its_kernels_is_captured():
-    """The engine's own choice (graphs=True): a repeating shape is measured once from its launch
-    list; here the kernels are so short that launching them takes the host longer than they run,
-    so the shape is captured and replayed (the opposite case, a model whose kernels outlast their
-    launches, is the 48-layer test of test_depth_gpu.py)."""
+    monkeypatch.setattr(engine_module, "launch_bound", verdict)
     model = model_for("A", "bfloat16")
     engine = bt.Engine(model, max_tokens=256)
     assert engine.use_graphs and engine.use_programs
@@ -152,8 +136,30 @@ def test_a_small_model_whose_launches_outlast_its_kernels_is_captured():
     rows = [engine.step([(slot, ids[:8])], want=[list(range(8))]).clone()]
     for t in range(8, 40):
         rows.append(engine.step([(slot, [ids[t]])]).clone())
-    # the shape's first step records its list, the second runs from it and is timed, the third reads the
-    # timing, captures and replays
-    assert engine.graphs_declined == 0 and engine.graph_replays == 32 - 2
+    probes = engine_module._PROBES
+    assert len(seen) == 1 and len(seen[0]) == probes and all(gpu > 0 and host > 0 for gpu, host in seen[0])
+    if gpu_is_the_limit:
+        assert engine.graphs_declined == 1 and engine.graph_replays == 0 and engine.program_runs == 32 - 1
+    else:
+        # the first step records, the next are measured from the list, the rest are replayed
+        assert engine.graphs_declined == 0 and engine.graph_replays == 32 - 1 - probes and engine.program_runs == probes
+    want = plain_logits("A", ids)
+    assert float((torch.cat(rows).cpu().double() - want).abs().max()) <= tolerance("bfloat16", want)
+
+
+def test_the_engine_chooses_a_path_for_a_repeating_shape_by_itself():
+    """The same without a given verdict: whatever this machine's clocks say, the decision is taken
+    once, the steps run from the list or from a graph, and the logits are right."""
+    model = model_for("A", "bfloat16")
+    engine = bt.Engine(model, max_tokens=256)
+    ids = prompts_for("A", [40], seed=87)[0]
+    slot = engine.open()
+    rows = [engine.step([(slot, ids[:8])], want=[list(range(8))]).clone()]
+    for t in range(8, 40):
+        rows.append(engine.step([(slot, [ids[t]])]).clone())
+    decisions = [v for v in engine._launch_bound.values() if isinstance(v, bool)]
+    assert len(decisions) == 1
+    assert engine.graph_replays + engine.program_runs == 32 - 1
+    assert (engine.graph_replays > 0) == (decisions[0] is False)
     want = plain_logits("A", ids)
     assert float((torch.cat(rows).cpu().double() - want).abs().max()) <= tolerance("bfloat16", want)

@@ -72,3 +72,19 @@ def test_context_classes():
     assert plan.context_limit == 4096 and plan.decode
     # never more than a sequence can hold (3 blocks of 64 tokens here)
     assert StepPlan([0], [100], [1], [5], [0], [[[0, 1]]], 3).context_limit == 192
+
+
+def test_whether_a_graph_pays_is_decided_by_the_median_of_the_measured_steps():
+    """``engine.launch_bound``: the GPU is the limit (no graph) when its time for a step stands
+    clearly above the host's time for walking the step's launch list; one odd sample of three
+    changes nothing."""
+    from burn_transformers_amd.engine.engine import launch_bound
+    host_bound = (1.00e-3, 0.98e-3)       # the GPU waited for every launch: both times about equal
+    gpu_bound = (1.70e-3, 1.30e-3)        # the kernels outlast their launches
+    assert launch_bound([gpu_bound] * 3) is True
+    assert launch_bound([host_bound] * 3) is False
+    assert launch_bound([gpu_bound, host_bound, gpu_bound]) is True
+    assert launch_bound([host_bound, (9e-3, 1e-3), host_bound]) is False      # a first use, a clock still rising
+    assert launch_bound([gpu_bound, (1e-3, 9e-3), gpu_bound]) is True         # the host was interrupted once
+    assert launch_bound([(1.05e-3, 1e-3)]) is False and launch_bound([(1.2e-3, 1e-3)]) is True
+    assert launch_bound([(1e-3, 0.0)]) is True                                # never a division by zero

@@ -86,7 +86,7 @@ def test_64_unequal_prompts_in_chunks_of_256_then_sampled_at_temperature_1(dtype
                 assert token == plain.sample_index(z, 1.0, u) or min(u - low, float(c[token]) - u) < band
             error = abs(logp - plain.log_probability(z, token, 1.0))
             worst = max(worst, error)
-            assert error < (2e-4 if dtype == "float32" else 0.15), f"row {row} step {s}: log-probability off by {error}"
+            assert error < (1e-4 if dtype == "float32" else 6e-2), f"row {row} step {s}: log-probability off by {error}"
         print(f"[medium] {dtype} row {row}: {len(prompts[row])} prompt tokens, log-probabilities within {worst:.3g}", flush=True)
     if dtype == "float32":
         whole = bt.generate(engine, prompts, config, total_length=MEDIUM["n_positions"])

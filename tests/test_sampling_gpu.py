@@ -176,3 +176,68 @@ def test_sampled_generation_with_truncation_is_reproducible_and_respects_top_k()
     other = bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=12, strategy="sample", temperature=1.3,
                                                              top_k=20, top_p=0.95, min_p=0.01, repetition_penalty=1.1, seed=12))
     assert [s.token_ids for s in once] != [s.token_ids for s in other]
+
+
+def test_a_row_keeps_the_draws_of_its_place_in_the_batch_as_it_started():
+    """Three rows start together; the middle one ends after its first token.  The reference keeps
+    the finished row in the batch and reserves a draw for it in every selection
+    (src/generation.rs:667-699: one block of ``batch`` counters per call), so the third row goes on
+    with draws s * 3 + 2.  Had the draws been numbered by the rows still alive it would use
+    s * 2 + 1: in every step where the two candidate draws choose different tokens from the plain
+    implementation's distribution, the generated token is the first candidate's."""
+    name, seed = "A", 5
+    folder, config, weights = model_folder(name, 8.0)
+    model = bt.load_model(folder, dtype="float32", device=DEV)
+    engine = bt.Engine(model, max_tokens=1024)
+    prompts = prompts_for(name, [9, 30, 17], seed=61)
+    steps = 24
+    cfg = bt.GenerationConfig(max_new_tokens=steps, strategy="sample", temperature=1.0, seed=seed)
+    # the middle row may hold 31 tokens in all: it ends, by its length, with its first new token
+    out = bt.generate(engine, prompts, cfg, total_length=31)
+    assert [len(s.token_ids) for s in out] == [22, 1, 14]
+    separated = 0
+    for row, alive_index in ((0, 0), (2, 1)):
+        sequence = out[row]
+        logits = plain.forward(prompts[row] + sequence.token_ids, weights, config)
+        for s, token in enumerate(sequence.token_ids):
+            z = logits[len(prompts[row]) - 1 + s]
+            c = torch.cumsum(torch.softmax(z, -1), -1)
+            as_started = plain.interior_unit(plain.splitmix64(seed, s * 3 + row))
+            low = float(c[token - 1]) if token else 0.0
+            assert low - 1e-5 <= as_started <= float(c[token]) + 1e-5, f"row {row} step {s}"
+            if s == 0 or row == 0:
+                continue
+            by_alive_rows = plain.interior_unit(plain.splitmix64(seed, s * 2 + alive_index))
+            other = plain.sample_index(z, 1.0, by_alive_rows)
+            edge = min(abs(by_alive_rows - low), abs(by_alive_rows - float(c[token])))
+            if other != token and edge > 1e-4:
+                separated += 1
+    assert separated >= 8, f"only {separated} steps tell the two numberings apart"
+
+
+def test_the_log_probability_of_a_sampled_token_is_that_of_the_tempered_distribution():
+    """Logits ln 1, ln 2, ln 3, ln 4 (then nothing: -inf would be a probability of 0 as well, here the
+    vocabulary simply ends) at temperature 0.5 are probabilities 1, 4, 9, 16 over 30, so the chosen
+    token's log-probability is ln(k^2 / 30) where the raw distribution would give ln(k / 10): the
+    two differ by ln(k / 3), worked by hand, and greedy selection reports the raw one
+    (src/generation.rs:732-743: the log-softmax of the PROCESSED logits, and temperature is part of
+    the processing only when sampling, :35-37)."""
+    vocab = 4
+    rows = 64
+    z = torch.log(torch.arange(1, vocab + 1, dtype=torch.float32)).repeat(rows, 1).to(DEV)
+    config = bt.GenerationConfig(max_new_tokens=1, strategy="sample", temperature=0.5, seed=123)
+    sampler = bt.Sampler(config, rows, torch.device(DEV), vocab)
+    ids, logps = sampler.select(z, list(range(rows)))
+    edges = [0.0, 1 / 30, 5 / 30, 14 / 30, 1.0]
+    chosen = set()
+    for row, (token, logp) in enumerate(zip(ids, logps)):
+        u = plain.interior_unit(plain.splitmix64(123, row))
+        assert edges[token] - 1e-6 <= u <= edges[token + 1] + 1e-6, f"row {row}"
+        k = token + 1
+        assert abs(logp - math.log(k * k / 30)) < 1e-5
+        assert abs((logp - math.log(k / 10)) - math.log(k / 3)) < 1e-5      # tempered minus raw, by hand
+        chosen.add(token)
+    assert len(chosen) >= 3            # the draws reach most tokens, so every k above was exercised
+    greedy = bt.Sampler(bt.GenerationConfig(max_new_tokens=1, temperature=0.5), rows, torch.device(DEV), vocab)
+    ids, logps = greedy.select(z, list(range(rows)))
+    assert set(ids) == {3} and all(abs(logp - math.log(4 / 10)) < 1e-5 for logp in logps)

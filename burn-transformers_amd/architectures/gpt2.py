@@ -47,7 +47,7 @@ def plan(config: GPT2Config) -> ModelPlan:
         mixer = PartSpec("attention", {
             "width": width, "heads": config.n_head, "kv_heads": config.n_head,
             "head_dim": config.head_size, "scale": attention_scale(config, i),
-            "causal": config.causal, "window": 0, "position": None},
+            "causal": config.causal, "window": 0},
             {"qkv_weight": p + "attn.c_attn.weight", "qkv_bias": p + "attn.c_attn.bias",
              "out_weight": p + "attn.c_proj.weight", "out_bias": p + "attn.c_proj.bias"})
         feed_forward = PartSpec("dense", {

@@ -44,8 +44,8 @@ class CausalLM:
         # a step of this model can be kept as a launch list if every part only launches kernels
         self.recordable = all(block.recordable() for block in self.blocks) and \
             all(part.only_launches_kernels for part in (self.embedding, self.final_norm, self.readout))
-        head_dims = sorted({d for block in self.blocks for mixer in block.mixers() for d in mixer.head_dims()})
-        K.prepare(self.dtype, head_dims)
+        parts = [self.embedding, self.final_norm, self.readout] + [p for block in self.blocks for p in block.parts.values()]
+        K.prepare(self.dtype, sorted({name for part in parts for name in part.kernel_modules(self.dtype)}))
 
     def _check_schedule(self):
         """Every cache entry has exactly one writer, which runs before any reader, and readers keep

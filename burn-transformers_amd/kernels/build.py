@@ -19,7 +19,6 @@ import time
 PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
-HEADERS = ("common.h", "host.h", "epilogue.h", "attention.h", "calls.h", "no_alloc.h")
 # -packed-fp32-ops is switched off for every kernel: some packed 32-bit forms have produced
 # wrong values on this hardware generation.
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=" + ARCH, "-fPIC", "-shared",
@@ -27,35 +26,87 @@ FLAGS = ["-O3", "-std=c++17", "--offload-arch=" + ARCH, "-fPIC", "-shared",
 ATTENTION_HEAD_SIZES = tuple(range(16, 129, 16))
 
 
-def module_source(name):
-    """(source file, extra definitions) of a module name."""
-    if name.startswith("attention_bf16_hd"):
-        size = int(name[len("attention_bf16_hd"):])
-        if size not in ATTENTION_HEAD_SIZES:
+class ModuleSpec:
+    """One kernel module: a source file, the definitions and link options it is compiled with, and
+    headers of its own beside the package's (which every module may include)."""
+
+    def __init__(self, name, source, flags=(), headers=(), own=False):
+        self.name, self.source, self.flags, self.headers, self.own = name, source, tuple(flags), tuple(headers), own
+
+    def same_as(self, other):
+        return (self.source, self.flags, self.headers) == (other.source, other.flags, other.headers)
+
+
+_registered = {}
+_registry_lock = threading.Lock()
+
+
+def register_module(name, source, flags=(), headers=(), _own=False):
+    """Makes a kernel module known under ``name``: ``ensure`` compiles it when it is first needed,
+    ``build_all`` compiles it with the package's own, ``kernels.library`` loads it and types every
+    ``bt_*_call(stream, structure)`` entry point its source defines.  This is how a part brings
+    kernels of its own, without a change to the package.
+
+    source: the ``.hip`` / ``.cpp`` file (absolute, or relative to the package's ``csrc/``); it may
+    include the package's headers (``common.h``, ``host.h`` for error reporting, ``calls.h``, ...).
+    flags: definitions (``-DNAME=1``) and link options (``-lfoo``) beyond the package's own.
+    headers: further files the source includes; a change to any of them rebuilds the module.
+    Registering a name again with the same description is a no-op; with another it is an error."""
+    if not os.path.isabs(source):
+        source = os.path.join(CSRC_DIR, source)
+    spec = ModuleSpec(name, source, flags, [os.path.abspath(h) for h in headers], _own)
+    with _registry_lock:
+        held = _registered.get(name)
+        if held is not None and not held.same_as(spec):
+            raise ValueError(f"kernel module {name!r} is registered already, from {held.source}")
+        _registered[name] = held or spec
+    return _registered[name]
+
+
+def module_spec(name):
+    spec = _registered.get(name)
+    if spec is None:
+        if name.startswith("attention_bf16_hd"):
             raise ValueError(
-                f"no bfloat16 attention kernel for head size {size}: "
+                f"no bfloat16 attention kernel for head size {name[len('attention_bf16_hd'):]}: "
                 f"sizes {ATTENTION_HEAD_SIZES[0]}..{ATTENTION_HEAD_SIZES[-1]} in steps of 16 are built")
-        return "attention_bf16.hip", [f"-DBT_HEAD_DIM={size}"]
-    if name in ("core", "gemm_mfma", "attention_f32"):
-        return name + ".hip", []
-    if name == "gemm_library":      # host code around hipBLASLt, which it opens at run time
-        return name + ".hip", ["-ldl"]
-    if name == "program":           # the host loop that walks a launch list: C++ only, no kernels
-        return name + ".cpp", []
-    raise ValueError(f"unknown kernel module {name!r}")
+        raise ValueError(f"unknown kernel module {name!r}; registered: {sorted(_registered)}")
+    return spec
+
+
+def package_headers():
+    """Every header of the package's ``csrc/``: each is part of every module's hash."""
+    return sorted(os.path.join(CSRC_DIR, f) for f in os.listdir(CSRC_DIR) if f.endswith(".h"))
+
+
+def entry_points(name):
+    """The ``bt_*_call`` entry points a module's source defines (its launch-list forms)."""
+    import re
+    with open(module_spec(name).source, errors="replace") as handle:
+        return sorted(set(re.findall(r"\b(bt_\w+_call)\s*\(", handle.read())))
+
+
+# the package's own modules
+for _name in ("core", "gemm_mfma", "attention_f32"):
+    register_module(_name, _name + ".hip", _own=True)
+register_module("gemm_library", "gemm_library.hip", ["-ldl"], _own=True)   # host code around hipBLASLt, opened at run time
+register_module("program", "program.cpp", _own=True)                       # the host loop that walks a launch list
+for _size in ATTENTION_HEAD_SIZES:                                         # the bfloat16 attention, once per head size
+    register_module(f"attention_bf16_hd{_size}", "attention_bf16.hip", [f"-DBT_HEAD_DIM={_size}"], _own=True)
 
 
 def all_modules():
-    return ["core", "gemm_mfma", "gemm_library", "program", "attention_f32"] + [f"attention_bf16_hd{s}" for s in ATTENTION_HEAD_SIZES]
+    """Every registered module: the package's own and what parts have brought so far."""
+    return list(_registered)
 
 
 def _hash(name):
-    source, defs = module_source(name)
+    spec = module_spec(name)
     digest = hashlib.sha256()
-    for part in HEADERS + (source,):
-        with open(os.path.join(CSRC_DIR, part), "rb") as handle:
+    for path in package_headers() + list(spec.headers) + [spec.source]:
+        with open(path, "rb") as handle:
             digest.update(handle.read())
-    digest.update(" ".join(FLAGS + defs).encode())
+    digest.update(" ".join(FLAGS + list(spec.flags)).encode())
     return digest.hexdigest()
 
 
@@ -117,15 +168,15 @@ def hipcc():
 
 def compile_module(name, verbose=True):
     """Compiles one module and returns the path of its library."""
-    source, defs = module_source(name)
+    spec = module_spec(name)
     target_dir = next((d for d in lib_dirs() if _writable(d)), None)
     if target_dir is None:
         raise RuntimeError(f"no writable folder for compiled kernels among {lib_dirs()}")
     lib = os.path.join(target_dir, name + ".so")
     partial = os.path.join(target_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.so")
-    options = [d for d in defs if not d.startswith("-l")]
-    libraries = [d for d in defs if d.startswith("-l")]
-    command = [hipcc()] + FLAGS + options + ["-o", partial, os.path.join(CSRC_DIR, source)] + libraries
+    options = [d for d in spec.flags if not d.startswith("-l")]
+    libraries = [d for d in spec.flags if d.startswith("-l")]
+    command = [hipcc()] + FLAGS + ["-I", CSRC_DIR] + options + ["-o", partial, spec.source] + libraries
     if verbose:
         print(f"[burn_transformers_amd] compiling {name} for {ARCH} ...", file=sys.stderr, flush=True)
     started = time.time()
@@ -174,7 +225,7 @@ def ensure_many(names, verbose=True, jobs=8):
 
 
 def build_all(verbose=True, jobs=8):
-    """Compiles every module anew (the build check of the repository)."""
+    """Compiles every registered module anew (the build check of the repository)."""
     from concurrent.futures import ThreadPoolExecutor
     names = all_modules()
     with ThreadPoolExecutor(max_workers=jobs) as pool:

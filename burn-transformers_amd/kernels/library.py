@@ -162,10 +162,8 @@ class Normalized:
 
 
 # Every kernel of a step is called through its structure form, bt_<kernel>_call(stream, structure)
-# (csrc/calls.h): the same pair can be called now or kept in a launch list (:class:`Program`).
-_CALLS = ("bt_embed_call", "bt_add_norm_call", "bt_gemm_plain_call", "bt_gemm_tile_call", "bt_gemm_skinny_call",
-          "bt_gemm_library_call", "bt_attention_plain_call", "bt_attention_f32_call",
-          "bt_attention_prefill_bf16_call", "bt_attention_decode_bf16_call", "bt_kv_copy_call")
+# (csrc/calls.h): the same pair can be called now or kept in a launch list (:class:`Program`).  A
+# module's entry points of that form are found in its source when it is loaded (``build.entry_points``).
 
 _modules = {}
 _lock = threading.Lock()
@@ -183,9 +181,9 @@ def _module(name):
                 lib = ctypes.CDLL(path)
             except OSError as error:
                 raise RuntimeError(f"cannot load the kernel library {path}: {error}") from error
-            if name != "program":
+            if hasattr(lib, "bt_last_error"):
                 lib.bt_last_error.restype = ctypes.c_char_p
-            for entry in _CALLS:
+            for entry in build.entry_points(name):
                 if hasattr(lib, entry):
                     getattr(lib, entry).argtypes = [_c_ptr, _c_ptr]
             _modules[name] = lib
@@ -194,7 +192,19 @@ def _module(name):
 
 def _check(lib, code):
     if code != 0:
-        raise KernelError(lib.bt_last_error().decode())
+        raise KernelError(lib.bt_last_error().decode() if hasattr(lib, "bt_last_error")
+                          else f"a kernel module's entry point returned {code}")
+
+
+register_module = build.register_module      # how a part brings kernels of its own: see there
+
+
+def launch(module, entry, call):
+    """Calls ``entry`` (an entry point ``int bt_*_call(void* stream, const Structure*)``) of the
+    registered module ``module`` with the ctypes structure ``call``, on the current stream: now,
+    or, while a launch list is being recorded, as one more call of that list.  The structure must
+    name only addresses that stay where they are (weights, the step's workspaces and tables)."""
+    _launch(_module(module), entry, call)
 
 
 class _Recorder(threading.local):
@@ -266,7 +276,8 @@ class Program:
         code = runner.bt_program_run(_c_ptr(_stream()), self._entries, _c_int(len(self.calls)), ctypes.byref(failed))
         if code != 0:
             lib, name, _ = self.calls[failed.value]
-            raise KernelError(f"{lib.bt_last_error().decode()} (call {failed.value} of {len(self.calls)}, {name})")
+            message = lib.bt_last_error().decode() if hasattr(lib, "bt_last_error") else f"returned {code}"
+            raise KernelError(f"{message} (call {failed.value} of {len(self.calls)}, {name})")
 
 
 class _Recording:
@@ -323,15 +334,13 @@ def require_gpu():
                            "there is no CPU path")
 
 
-def prepare(dtype, head_dims=()):
-    """Builds and loads what a model of this dtype and these head sizes needs."""
+def prepare(dtype, modules=()):
+    """Builds and loads what every model of this dtype needs, and the modules its parts ask for
+    (``Part.kernel_modules``)."""
     names = ["core", "gemm_mfma", "program"]
-    if dtype == torch.bfloat16:
-        if os.environ.get(PRODUCTS_ENV, "") != "own":
-            names.append("gemm_library")
-        names += [f"attention_bf16_hd{size}" for size in head_dims]
-    elif any(size <= 128 and size % 16 == 0 for size in head_dims):
-        names.append("attention_f32")
+    if dtype == torch.bfloat16 and os.environ.get(PRODUCTS_ENV, "") != "own":
+        names.append("gemm_library")
+    names += [name for name in modules if name not in names]
     with _lock:
         build.ensure_many(names)        # what is missing is compiled side by side
     for name in names:

@@ -79,8 +79,12 @@ class CausalSelfAttention(Mixer):
     def kv_spec(self):
         return KVSpec(self.kv_heads, self.head_dim, self.window)
 
-    def head_dims(self):
-        return () if self.plain_only else (self.head_dim,)
+    def kernel_modules(self, dtype):
+        if self.plain_only:
+            return ()
+        if dtype == torch.bfloat16:
+            return (f"attention_bf16_hd{self.head_dim}",)
+        return ("attention_f32",) if self.head_dim <= 128 else ()
 
     def decode_runs(self, step, device):
         """Into how many runs a decode step's keys are cut: planned for the step's class of

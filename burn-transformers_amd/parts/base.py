@@ -104,6 +104,12 @@ class Part:
     def __init__(self, params, tensors):
         self.params, self.tensors = params, tensors
 
+    def kernel_modules(self, dtype):
+        """Names of kernel modules (``kernels.build.register_module``) that must be built and loaded
+        before this part's first step, beyond those every model uses: what the part's own kernels
+        live in.  They are compiled side by side when the model is built."""
+        return ()
+
 
 class Norm(Part):
     def apply(self, stream, step, rows=None):
@@ -145,10 +151,6 @@ class Mixer(Part):
 
     def state_spec(self):
         return None
-
-    def head_dims(self):
-        """Head sizes for which attention kernels must be built."""
-        return ()
 
     def forward(self, h, step, memory, stream):
         """Adds the mixer's contribution to ``stream`` (or returns it as a Delta)."""

@@ -123,7 +123,7 @@ def test_attention_mixer_alone(dtype, heads, kv_heads, hd, width, window):
         {"width": width, "heads": heads, "kv_heads": kv_heads, "head_dim": hd, "scale": scale, "window": window},
         {"qkv_weight": qkv_w.to(DEV), "qkv_bias": qkv_b.to(DEV), "out_weight": out_w.to(DEV), "out_bias": out_b.to(DEV)})
     assert mixer.kv_spec() == KVSpec(kv_heads, hd, window)
-    bt.kernels.library.prepare(dt, mixer.head_dims())
+    bt.kernels.library.prepare(dt, mixer.kernel_modules(dt))
     cache = Cache([mixer.kv_spec()], [None], max_tokens=512, max_sequence_length=256, dtype=dt, device=DEV)
     lengths = [90, 7]
     xs = [rnd(gen, n, width).to(dt) for n in lengths]

@@ -5,7 +5,9 @@
   x + mixer(norm(x)) + feed_forward(norm(x));
 * a block without any mixer (norm and feed-forward only), which has no cache entry;
 * a mixer with a position encoding of its own: it rotates queries and keys by their positions
-  before the keys go into the cache (the token table gets no positions at all).
+  before the keys go into the cache (the token table gets no positions at all), with a kernel
+  file of its own (``tests/toy_kernels/rotary_turn.hip``) that the package's build compiles and
+  whose calls go into launch lists like the package's own.
 
 The engine asks a block which of its parts mix tokens (``Block.mixers``) and what a run of it
 keeps (``Block.cache_needs``); it knows no part by name."""
@@ -23,10 +25,12 @@ from burn_transformers_amd.cache.storage import KVSpec  # noqa: E402
 from burn_transformers_amd.engine.plan import LayerPlan, ModelPlan, PartSpec, ScheduleEntry  # noqa: E402
 from burn_transformers_amd.kernels import library as K  # noqa: E402
 from burn_transformers_amd.parts import Block, Mixer, register, unregister  # noqa: E402
+import toy_kernels  # noqa: E402
 
 
 class SideBySideBlock(Block):
     ROLES = {"norm": "norm", "tokens": "mixer", "channels": "feed_forward"}
+    only_launches_kernels = True
 
     def forward(self, stream, step, memory):
         h = self.parts["norm"].apply(stream, step)
@@ -38,6 +42,7 @@ class SideBySideBlock(Block):
 
 class ChannelsOnlyBlock(Block):
     ROLES = {"norm": "norm", "channels": "feed_forward"}
+    only_launches_kernels = True
 
     def forward(self, stream, step, memory):
         assert memory is None
@@ -48,7 +53,11 @@ class ChannelsOnlyBlock(Block):
 
 class RotatingAttention(Mixer):
     """Attention whose queries and keys are turned by their positions: channel pair (i, i + h/2) of
-    a head by the angle pos * base^(-2i/h), computed in float32; keys are cached turned."""
+    a head by the angle pos * base^(-2i/h), computed in float32; keys are cached turned.  The turn
+    is a kernel this test brings (``toy_kernels``): the part asks for its module by name, and does
+    nothing in a step but launch kernels, so its steps are kept as launch lists."""
+
+    only_launches_kernels = True
 
     def __init__(self, params, tensors):
         super().__init__(params, tensors)
@@ -62,27 +71,21 @@ class RotatingAttention(Mixer):
     def kv_spec(self):
         return KVSpec(self.heads, self.head_dim, 0)
 
-    def head_dims(self):
-        return (self.head_dim,)
-
-    def turn(self, rows, positions):
-        tokens = rows.shape[0]
-        x = rows.float().view(tokens, self.heads, 2, self.head_dim // 2)
-        angle = positions.float()[:, None] * self.freq[None, :]
-        cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
-        first, second = x[:, :, 0], x[:, :, 1]
-        turned = torch.stack([first * cos - second * sin, second * cos + first * sin], dim=2)
-        return turned.reshape(tokens, self.width).to(rows.dtype)
+    def kernel_modules(self, dtype):
+        attention = f"attention_bf16_hd{self.head_dim}" if dtype == torch.bfloat16 else "attention_f32"
+        return [attention] + toy_kernels.register()
 
     def forward(self, h, step, memory, stream):
         tokens, d = h.shape[0], self.width
         qkv = step.buffer("toy.qkv", tokens, 3 * d, step.dtype)
         K.gemm(h, self.qkv, K.epilogue_store(qkv))
-        q, k = self.turn(qkv[:, :d], step.tok_pos), self.turn(qkv[:, d:2 * d], step.tok_pos)
+        K.launch("toy_rotary_turn", "bt_toy_rotary_turn_call", toy_kernels.RotaryTurnCall(
+            dtype=K.DTYPE_CODES[step.dtype], tokens=tokens, parts=2, heads=self.heads, head_dim=self.head_dim,
+            ld=qkv.stride(0), rows=qkv.data_ptr(), positions=step.tok_pos.data_ptr(), freq=self.freq.data_ptr()))
         kv = memory.kv()
-        K.kv_copy(k, qkv[:, 2 * d:].contiguous(), step.tok_seq, step.tok_pos, kv, to_cache=True)
+        K.kv_copy(qkv[:, d:2 * d], qkv[:, 2 * d:], step.tok_seq, step.tok_pos, kv, to_cache=True)
         mixed = step.buffer("toy.mixed", tokens, d, step.dtype)
-        K.attention(K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
+        K.attention(K.attention_args(qkv[:, :d], mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                      self.heads, step.n_seqs, step.max_count, self.head_dim ** -0.5), step.dtype, step.decode)
         stream.add_product(step, mixed, self.out)
 
@@ -218,6 +221,23 @@ def test_blocks_with_other_roles_no_mixer_and_a_turning_mixer(dtype, tmp_path):
                 engine.close(slot)
         assert engine.graph_replays >= 8
         engine.cache.ledger.check()
+        # The model only launches kernels (the toy's own among them), so its steps are kept as launch
+        # lists: walked in C++ they give the bits that the same calls give one by one from Python.
+        assert model.recordable and "toy_rotary_turn" in K.loaded_modules()
+        listed = bt.Engine(model, max_tokens=1024, graphs=False)
+        direct = bt.Engine(model, max_tokens=1024, graphs=False, programs=False)
+        assert listed.use_programs and not direct.use_programs
+        for round_ in range(2):                 # the second round's shapes are walked from their lists
+            pairs = [(listed.open(), direct.open()) for _ in requests]
+            for begin, end in ((0, 5), (5, 6), (6, 7), (7, 9)):
+                a = listed.step([(p[0], r[begin:end]) for p, r in zip(pairs, requests)]).clone()
+                b = direct.step([(p[1], r[begin:end]) for p, r in zip(pairs, requests)]).clone()
+                assert torch.equal(a, b), f"round {round_} tokens {begin}..{end}"
+            assert any(name == "bt_toy_rotary_turn_call" for _, name, _ in listed.last_program.calls)
+            for a, b in pairs:
+                listed.close(a)
+                direct.close(b)
+        assert listed.program_runs >= 5 and direct.program_runs == 0
     finally:
         unregister("block", "toy_side_by_side")
         unregister("block", "toy_channels_only")

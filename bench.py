@@ -1,7 +1,8 @@
 """Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
-                    [--repetitions 10] [--workload xl|small|medium|sweep] [--no-points] [--no-kernels] [--no-own]
+                    [--repetitions 10] [--workload xl|small|medium|sweep] [--model xl|medium|small]
+                    [--kernel-batches 1,64] [--no-points] [--no-kernels] [--no-own]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
 sequences, prefilled with 512 synthetic tokens each, is decoded towards 1,024.  A step is one
@@ -24,12 +25,18 @@ One JSON line is printed:
               products to its backend's library)
   roofline    bytes a decode step has to read (every weight once + the live cache) / its time,
               against 8 TB/s
-  points      decoded tokens per second at batch 1 and 64
+  points      decoded tokens per second at batch 1 and 64, at batch 8 from prompts of 896 tokens
+              (contexts up to the position limit), and prompt tokens per second of 2 x 1,024
+              prompt tokens fed in chunks of 256 (eight steps of 2 x 256 tokens)
   kernels     for the decode step and for the prefill step, each class of kernel on its own: the
               step's launch list is cut into classes (same kernel, same shape), each class's calls
               (one per layer, every layer's own weights) are replayed alone from a HIP graph and
               timed with events; per call: microseconds and the fraction of the HBM roofline
               (decode) or of the MFMA peak (prefill)
+
+``--model medium`` / ``--model small`` run the same measurement (same JSON line) at the layer sizes
+of GPT-2 medium and small; ``--kernel-batches 1,64`` adds the kernel classes of decode steps of
+those batch sizes beside the main one (``kernels.decode_b1`` ...).
 
 ``--workload small`` and ``--workload medium`` run the other two measured workloads through the
 generation loop: GPT-2 small sizes in float32, 16 prompts of 1 to 1,000 tokens decoded greedily to
@@ -54,6 +61,8 @@ XL = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 48,
       "layer_norm_epsilon": 1e-5}
 SMALL = dict(XL, n_layer=12, n_embd=768, n_head=12, n_inner=3072)
 MEDIUM = dict(XL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
+MODELS = {"xl": XL, "medium": MEDIUM, "small": SMALL}
+MODEL_NAMES = {"xl": "XL", "medium": "medium", "small": "small"}
 PROMPT_LEN, CONTEXT_LEN, PREFILL_SEQS, PREFILL_LEN = 512, 1024, 2, 1024
 WARMUP_REPETITIONS = 3
 
@@ -81,13 +90,14 @@ def synthetic_prompts(batch, length, vocab, seed):
     return torch.randint(0, vocab, (batch, length), generator=gen).tolist()
 
 
-def decode_repetition(engine, batch, warmup, steps, vocab, seed):
+def decode_repetition(engine, batch, warmup, steps, vocab, seed, prompt_len=PROMPT_LEN):
     """One repetition on fresh sequences: (seconds of the timed steps, first context length)."""
     import torch
 
     import burn_transformers_amd as bt
+    from burn_transformers_amd.engine.generate import select_and_step_ahead
     from burn_transformers_amd.sampling.sampler import Sampler
-    prompts = synthetic_prompts(batch, PROMPT_LEN, vocab, seed=seed)
+    prompts = synthetic_prompts(batch, prompt_len, vocab, seed=seed)
     slots = [engine.open() for _ in prompts]
     sampler = Sampler(bt.GenerationConfig(), batch, engine.device)
     rows = list(range(batch))
@@ -96,46 +106,43 @@ def decode_repetition(engine, batch, warmup, steps, vocab, seed):
     for begin in range(0, batch, 8):
         part = engine.step([(slots[i], prompts[i]) for i in range(begin, min(begin + 8, batch))])
         logits[begin:begin + part.shape[0]] = part
-    sampler.launch(logits, rows)
-    entries = [(slot, [0]) for slot in slots]
 
-    def one_step():
-        # as the generation loop decodes: the chosen ids feed the step from the GPU, and the host
-        # reads them (the step's one readback) while the step runs
-        logits = engine.step(entries, device_tokens=sampler.device_ids(batch))
-        sampler.result()
-        sampler.launch(logits, rows)
+    def run(count, logits):
+        # the generation loop's own turn: the selection is started, its ids feed the next step from
+        # the GPU, and the host reads them (the step's one readback) while that step runs
+        for _ in range(count):
+            _, _, logits = select_and_step_ahead(engine, sampler, slots, logits, rows, rows)
+        return logits
 
-    for _ in range(warmup):
-        one_step()
+    logits = run(warmup, logits)
     first_context = engine.length(slots[0])
     torch.cuda.synchronize()
     started = time.perf_counter()
-    for _ in range(steps):
-        one_step()
+    run(steps, logits)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
-    sampler.result()
     for slot in slots:
         engine.close(slot)
     return elapsed, first_context
 
 
-def decode_run(engine, batch, warmup, steps, vocab, repetitions, warmup_repetitions=WARMUP_REPETITIONS):
+def decode_run(engine, batch, warmup, steps, vocab, repetitions, warmup_repetitions=WARMUP_REPETITIONS,
+               prompt_len=PROMPT_LEN):
     """(sorted seconds of the measured repetitions, steps, mean context length over the timed steps)."""
-    steps = max(1, min(steps, CONTEXT_LEN - PROMPT_LEN - warmup - 1))
+    steps = max(1, min(steps, CONTEXT_LEN - prompt_len - warmup - 1))
     for r in range(warmup_repetitions):          # short: they are there for graphs, clocks and caches
-        decode_repetition(engine, batch, warmup, min(steps, 24), vocab, seed=1000 + r)
-    times, first_context = [], PROMPT_LEN
+        decode_repetition(engine, batch, warmup, min(steps, 24), vocab, 1000 + r, prompt_len)
+    times, first_context = [], prompt_len
     for r in range(repetitions):
-        elapsed, first_context = decode_repetition(engine, batch, warmup, steps, vocab, seed=batch * 100 + r)
+        elapsed, first_context = decode_repetition(engine, batch, warmup, steps, vocab, batch * 100 + r, prompt_len)
         times.append(elapsed)
     mean_context = first_context + (steps + 1) / 2.0     # keys each step's query reads, itself included
     return sorted(times), steps, mean_context
 
 
-def prefill_run(engine, vocab, repetitions):
-    """Sorted seconds of one step of PREFILL_SEQS x PREFILL_LEN prompt tokens on fresh sequences."""
+def prefill_run(engine, vocab, repetitions, chunk=None):
+    """Sorted seconds of PREFILL_SEQS x PREFILL_LEN prompt tokens on fresh sequences: in one step, or
+    in steps of ``chunk`` tokens of every sequence."""
     import torch
     times = []
     for r in range(WARMUP_REPETITIONS + repetitions):
@@ -143,7 +150,8 @@ def prefill_run(engine, vocab, repetitions):
         slots = [engine.open() for _ in prompts]
         torch.cuda.synchronize()
         started = time.perf_counter()
-        engine.step(list(zip(slots, prompts)))
+        for begin in range(0, PREFILL_LEN, chunk or PREFILL_LEN):
+            engine.step([(slot, prompt[begin:begin + (chunk or PREFILL_LEN)]) for slot, prompt in zip(slots, prompts)])
         torch.cuda.synchronize()
         times.append(time.perf_counter() - started)
         for slot in slots:
@@ -275,7 +283,7 @@ def run_xl(args):
     import burn_transformers_amd as bt
     from burn_transformers_amd.kernels import library as K
 
-    config = dict(XL, n_layer=args.layers)
+    config = dict(MODELS[args.model], n_layer=args.layers)
     model = build_model(config, args.dtype)
     vocab = config["vocab_size"]
     weight_bytes, kv_per_token, prefill_flops = model_bytes_and_flops(config, args.layers, args.dtype)
@@ -300,6 +308,8 @@ def run_xl(args):
     kernels = {}
     if not args.no_kernels:
         kernels["decode"] = decode_kernels(engine, args.batch, vocab, config, args.dtype, int(mean_context))
+        for batch in args.kernel_batches:
+            kernels[f"decode_b{batch}"] = decode_kernels(engine, batch, vocab, config, args.dtype, int(mean_context))
         kernels["prefill"] = prefill_kernels(engine, vocab, config, args.dtype)
     if args.dtype == "bf16" and K.library_products() is not None and not args.no_own:
         # the same step with every product on this package's own kernels
@@ -319,14 +329,20 @@ def run_xl(args):
         for batch in (1, 64):
             t, s, _ = decode_run(engine, batch, args.warmup, args.steps, vocab, max(3, args.repetitions // 2), 1)
             points[f"decode_b{batch}"] = round(batch * s / statistics.median(t), 1)
+        # contexts near the position limit: batch 8 from prompts of 896 tokens towards 1,024
+        t, s, _ = decode_run(engine, 8, args.warmup, args.steps, vocab, max(3, args.repetitions // 2), 1, prompt_len=896)
+        points["decode_b8_from896"] = round(8 * s / statistics.median(t), 1)
+        # the same 2 x 1,024 prompt tokens as `prefill`, fed in chunks of 256 tokens of each sequence
+        chunked = statistics.median(prefill_run(engine, vocab, max(3, args.repetitions // 2), chunk=256))
+        points["prefill_2x1024_chunks256"] = round(PREFILL_SEQS * PREFILL_LEN / chunked, 1)
 
     return {
-        "metric": f"decode tok/s at batch {args.batch} (GPT-2 XL sizes, 512-token prompts decoded to "
+        "metric": f"decode tok/s at batch {args.batch} (GPT-2 {MODEL_NAMES[args.model]} sizes, 512-token prompts decoded to "
                   f"{final_context} tokens, median of {args.repetitions} repetitions)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic token ids, random weights",
-        "config": {"model": "gpt2-xl", "n_layer": args.layers, "n_layer_full": XL["n_layer"],
+        "config": {"model": "gpt2-" + args.model, "n_layer": args.layers, "n_layer_full": MODELS[args.model]["n_layer"],
                    "n_embd": config["n_embd"], "n_head": config["n_head"], "n_inner": config["n_inner"],
                    "vocab_size": vocab, "n_positions": config["n_positions"], "global_batch": args.batch,
                    "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LEN, "final_context": final_context,
@@ -458,7 +474,10 @@ def main():
     parser.add_argument("--steps", type=int, default=CONTEXT_LEN - PROMPT_LEN - 16 - 1)
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--layers", type=int, default=XL["n_layer"], help="fewer layers than the 48 of GPT-2 XL")
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (48 for GPT-2 XL)")
+    parser.add_argument("--model", choices=sorted(MODELS), default="xl",
+                        help="whose layer sizes the default workload runs at: GPT-2 XL, medium or small")
+    parser.add_argument("--kernel-batches", default="", help="further batch sizes whose decode kernel classes are timed, e.g. 1,64")
     parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
     parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
     parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep"], default="xl")
@@ -471,6 +490,9 @@ def main():
         sys.exit(2)
     if args.repetitions < 1:
         parser.error("--repetitions must be at least 1")
+    args.kernel_batches = [int(b) for b in args.kernel_batches.split(",") if b]
+    if args.layers is None:
+        args.layers = XL["n_layer"] if args.workload == "sweep" else MODELS[args.model]["n_layer"]
     if args.workload == "sweep":
         run_sweep(args)
     elif args.workload == "xl":

@@ -119,29 +119,42 @@ def generate_batch(engine, prompts, config, prefill_chunk=None, on_token=None, l
     return tracker.sequences
 
 
+def select_and_step_ahead(engine, sampler, slots, logits, live, ahead):
+    """One turn of the decode pipeline, with the host one step behind the GPU: starts the selection
+    of one token for every row of ``live`` from ``logits``; feeds the rows of ``ahead`` (those of
+    ``live`` that go on unless this very token stops them, in the same order) their tokens straight
+    from the GPU (``Engine.step(device_tokens=...)``); only then waits for the selection's ids to
+    reach the host, while that step already runs.  Returns (ids, log-probabilities, the logits of
+    the step that was started for ``ahead``, or None if no row goes on).  The generation loop and
+    the benchmark both decode through this function."""
+    sampler.launch(logits, live)
+    next_logits = None
+    if ahead:
+        tokens = sampler.device_ids(len(live))
+        if len(ahead) != len(live):
+            going = set(ahead)
+            places = [i for i, row in enumerate(live) if row in going]
+            tokens = tokens[torch.tensor(places, device=engine.device)]
+        next_logits = engine.step([(slots[row], [0]) for row in ahead], device_tokens=tokens)
+    ids, logps = sampler.result()
+    return ids, logps, next_logits
+
+
 def _decode_ahead(engine, sampler, tracker, slots, open_rows, logits, live, on_token):
-    """The decode loop with the host one step behind the GPU.  A selection's ids stay on the GPU and
-    feed the next step from there (``Engine.step(device_tokens=...)``); the host reads them while
-    that step runs, so its own work (stop rules, the next step's tables) costs the GPU no idle
-    time.  A row whose token turns out to end it (end-of-sequence, a stop sequence) has then been
-    fed once too often: that position goes with the row's slot.  Rows that end by their length are
-    known beforehand and are not fed.  Tokens, log-probabilities and finish reasons are those of
-    the loop that waits for every token (the same kernels on the same rows; a row's logits do not
-    depend on what else is in the batch beyond rounding)."""
+    """The decode loop with the host one step behind the GPU (``select_and_step_ahead``): the host's
+    own work (stop rules, the next step's tables) costs the GPU no idle time.  A row whose token
+    turns out to end it (end-of-sequence, a stop sequence) has then been fed once too often: that
+    position goes with the row's slot.  Rows that end by their length are known beforehand and are
+    not fed.  Tokens, log-probabilities and finish reasons are those of the loop that waits for
+    every token up to rounding: a row that its token ends stays in the batch for one more step,
+    and the number of rows chooses the kernels of a step, so in bfloat16 the other rows' logits of
+    that one step may round differently than they would without it, and a near-tie may then choose
+    another token."""
     device = engine.device
     while True:
-        sampler.launch(logits, live)
         # rows that go on unless this very token stops them
         ahead = [row for row in live if len(tracker.sequences[row].token_ids) + 1 < tracker.limit(row)]
-        next_logits = None
-        if ahead:
-            tokens = sampler.device_ids(len(live))
-            if len(ahead) != len(live):
-                going = set(ahead)
-                places = [i for i, row in enumerate(live) if row in going]
-                tokens = tokens[torch.tensor(places, device=device)]
-            next_logits = engine.step([(slots[row], [0]) for row in ahead], device_tokens=tokens)
-        ids, logps = sampler.result()
+        ids, logps, next_logits = select_and_step_ahead(engine, sampler, slots, logits, live, ahead)
         next_live = []
         for row, token, logp in zip(live, ids, logps):
             if not math.isfinite(logp):

@@ -468,6 +468,139 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
   }
 }
 
+// The direct-to-LDS form again, for products of some tens to some hundreds of rows (short prompts,
+// chunks of prompts): a template over the tile (BM x BN, 64 or 128 each, four waves as 2 x 2) and
+// the number of stages.  Such a product has too few tiles of 128 x 128 to fill the chip, and with
+// smaller tiles a work-group has less arithmetic per byte it pulls, so that its time is the 25 (or
+// 100) trips to memory of its loop over K unless many of them are in flight at once: a tile of
+// 64 x 64 is 16 KiB a stage, and eight stages keep seven tiles (112 KiB) on their way while one is
+// multiplied.  Same layout of a stage as above (A's rows, then W's, 128 bytes each, the swizzle
+// applied on the memory side), same waits written by hand.  K a multiple of 64, operands below 4 GiB.
+// Measured at 128 rows (us; the vendor's library beside it): 4800 x 1600 12.0 (17.3), 6400 x 1600 13.6
+// (18.2), and with K cut into four slices of pending partial sums 1600 x 1600 6.7 (11.2), 1600 x 6400
+// 13.4 (18.4); at 256 rows tiles of 128 x 64 take 17.4 (20.0) and 20.0 (21.4), two slices of 64 x 64
+// 8.4 (11.7) and 20.6 (23.9); from 512 rows on the library wins.  What bounds these forms is their
+// loop of loads: with the matrix instructions and the LDS reads taken out the times stay (a
+// work-group gets a tile of 16 KiB every 0.4 us, whatever the number of stages), and a ring of
+// register sets in place of the direct loads was slower still.
+template <int NEWER, int LOADS>
+__device__ __forceinline__ void wait_for_all_but(int newer) {
+  // waits until at most `newer` tiles' loads (LOADS instructions each) of this wave are in flight
+  if constexpr (NEWER == 0) {
+    wait_vmcnt<0>();
+  } else {
+    if (newer >= NEWER) wait_vmcnt<NEWER * LOADS>();
+    else wait_for_all_but<NEWER - 1, LOADS>(newer);
+  }
+}
+
+template <int BM, int BN, int STAGES>
+__global__ void __launch_bounds__(256)
+gemm_tile_deep_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int M, int N,
+                      int K, Epilogue epi, int tiles_m, int tiles_n) {
+  constexpr int ROWS = BM + BN;                   // rows of a stage
+  constexpr int STAGE_BYTES = ROWS * TILE_ROW_BYTES;
+  constexpr int LOADS = ROWS / 32;                // global_load_lds instructions per wave and tile (8 rows each)
+  constexpr int TM = BM / 64, TN = BN / 64;       // 32-wide MFMA blocks of a wave's (BM / 2) x (BN / 2)
+  static_assert((BM == 64 || BM == 128) && (BN == 64 || BN == 128) && STAGES >= 3 && LOADS * (STAGES - 2) < 64,
+                "tiles of 64 or 128, and no more loads in flight than the wave's counter holds");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [STAGES][ROWS][128 bytes]
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int tile = xcd_contiguous(blockIdx.x, tiles_m * tiles_n);
+  const int m_base = (tile % tiles_m) * BM, n_base = (tile / tiles_m) * BN;
+  const int split = blockIdx.z, splits = gridDim.z;
+  const int k_tiles = K / TILE_K;
+  const int kt_begin = (int)((int64_t)k_tiles * split / splits);
+  const int count = (int)((int64_t)k_tiles * (split + 1) / splits) - kt_begin;
+
+  // load j of wave w fills stage rows 8 (LOADS w + j) .. + 7: A's rows below BM, W's from there on
+  const unsigned char* a_bytes = reinterpret_cast<const unsigned char*>(A) + (int64_t)kt_begin * (TILE_K * 2);
+  const unsigned char* w_bytes = reinterpret_cast<const unsigned char*>(W) + (int64_t)kt_begin * (TILE_K * 2);
+  unsigned off[LOADS];
+  bool from_w[LOADS];
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) {
+    int first_row = __builtin_amdgcn_readfirstlane(8 * (LOADS * wave + j));
+    from_w[j] = first_row >= BM;                  // (the same for the whole wave: eight rows never straddle BM)
+    int stage_row = first_row + (lane >> 3);
+    int chunk = (lane & 7) ^ ((stage_row >> 1) & 7);
+    int row = from_w[j] ? n_base + stage_row - BM : m_base + stage_row;
+    int limit = from_w[j] ? N : M;
+    row = row < limit ? row : limit - 1;
+    off[j] = (unsigned)(((int64_t)row * (from_w[j] ? (int64_t)K : lda) + chunk * 8) * 2);
+  }
+  auto issue = [&](int stage) {   // the tile a_bytes / w_bytes point at, into `stage`; then advance
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)((from_w[j] ? w_bytes : a_bytes) + off[j]),
+          (__attribute__((address_space(3))) void*)(lds + stage * STAGE_BYTES + 8 * (LOADS * wave + j) * TILE_ROW_BYTES),
+          16, 0, 0);
+    a_bytes += TILE_K * 2;
+    w_bytes += TILE_K * 2;
+  };
+  int w_rd[4], a_rd[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    w_rd[kk] = BM * TILE_ROW_BYTES + swizzled(wn * (BN / 2) + l32, 2 * kk + g);
+    a_rd[kk] = swizzled(wm * (BM / 2) + l32, 2 * kk + g);
+  }
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int bn = 0; bn < TN; ++bn)
+#pragma unroll
+    for (int bm = 0; bm < TM; ++bm)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[bn][bm][r] = 0.f;
+
+#pragma unroll
+  for (int t = 0; t < STAGES - 1; ++t)
+    if (t < count) issue(t);
+  int stage = 0, next_stage = STAGES - 1;
+  for (int i = 0; i < count; ++i) {
+    // tiles i + 1 .. i + STAGES - 2 (those that exist) may still be in flight
+    wait_for_all_but<STAGES - 2, LOADS>(count - 1 - i);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (i + STAGES - 1 < count) issue(next_stage);
+    const unsigned char* base = lds + stage * STAGE_BYTES;
+    bf16x8 wop[4][TN], aop[4][TM];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+      for (int b = 0; b < TN; ++b) wop[kk][b] = *reinterpret_cast<const bf16x8*>(base + w_rd[kk] + b * 4096);
+#pragma unroll
+      for (int b = 0; b < TM; ++b) aop[kk][b] = *reinterpret_cast<const bf16x8*>(base + a_rd[kk] + b * 4096);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int bn = 0; bn < TN; ++bn)
+#pragma unroll
+        for (int bm = 0; bm < TM; ++bm)
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wop[kk][bn], aop[kk][bm], acc[bn][bm], 0, 0, 0);
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+    next_stage = next_stage + 1 == STAGES ? 0 : next_stage + 1;
+  }
+
+  // lane holds D[i][j]: i = 8 * (r / 4) + 4 * g + r % 4 (column n), j = lane % 32 (row m)
+#pragma unroll
+  for (int bm = 0; bm < TM; ++bm) {
+    const int m = m_base + wm * (BM / 2) + bm * 32 + l32;
+#pragma unroll
+    for (int bn = 0; bn < TN; ++bn) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float v[4] = {acc[bn][bm][4 * q], acc[bn][bm][4 * q + 1], acc[bn][bm][4 * q + 2], acc[bn][bm][4 * q + 3]};
+        int n0 = n_base + wn * (BN / 2) + bn * 32 + q * 8 + g * 4;
+        if (m < M) epilogue4<bf16_t>(epi, N, m, n0, v, split);
+      }
+    }
+  }
+}
+
 // Memory latency on this GPU is about a microsecond and one compute unit alone pulls only a few
 // per cent of the HBM bandwidth, while a decode step is hundreds of short kernels.  So the
 // skinny kernel (a) wants at least as many work-groups as there are compute units, which is
@@ -720,10 +853,39 @@ static void launch_tile(hipStream_t stream, const T* A, int64_t lda, const T* W,
                      K, epi, tiles_m, tiles_n);
 }
 
+template <int BM, int BN, int STAGES>
+static int launch_deep_form(hipStream_t s, const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K,
+                            const Epilogue& epi, int splits) {
+  auto kernel = gemm_tile_deep_kernel<BM, BN, STAGES>;
+  const size_t lds = (size_t)STAGES * (BM + BN) * TILE_ROW_BYTES;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) BT_REFUSE("gemm_tile: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));
+    raised = true;
+  }
+  int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, 1, splits), dim3(256), lds, s, a, lda, w, M, N, K, epi, tiles_m, tiles_n);
+  return bt_check_launch("gemm_tile");
+}
+
+// variants 4 .. 7: the deep forms (64 x 64 with 8 or 4 stages, 128 x 64 with 6 or 3)
+static int launch_deep(hipStream_t s, int variant, const bf16_t* a, int64_t lda, const bf16_t* w, int M, int N, int K,
+                       const Epilogue& epi, int splits) {
+  switch (variant) {
+    case 4: return launch_deep_form<64, 64, 8>(s, a, lda, w, M, N, K, epi, splits);
+    case 5: return launch_deep_form<64, 64, 4>(s, a, lda, w, M, N, K, epi, splits);
+    case 6: return launch_deep_form<128, 64, 6>(s, a, lda, w, M, N, K, epi, splits);
+    case 7: return launch_deep_form<128, 64, 3>(s, a, lda, w, M, N, K, epi, splits);
+  }
+  BT_REFUSE("gemm_tile: unknown form %d", variant);
+}
+
 // dtype: 0 float, 1 bfloat16 (the codes of every entry point that takes both).
-// variant: 0 = the fastest form the operands allow; 1 = template, 2 = lean, 3 = direct to LDS
-// (asked for by tests and measurements; a form that cannot take the operands is refused; float
-// has the template only)
+// variant: 0 = the fastest form the operands allow; 1 = template, 2 = lean, 3 = direct to LDS,
+// 4 .. 7 = direct to LDS with smaller tiles and more stages (asked for by tests, by measurements
+// and, for steps of some tens to some hundreds of rows, by the caller; a form that cannot take
+// the operands is refused; float has the template only)
 BT_EXPORT int bt_gemm_tile(void* stream, int dtype, const void* A, int64_t lda, const void* W, int M, int N, int K,
                            const Epilogue* epi, int splits, int variant) {
   if (M <= 0) return BT_OK;
@@ -746,6 +908,7 @@ BT_EXPORT int bt_gemm_tile(void* stream, int dtype, const void* A, int64_t lda, 
   if (variant == 0) variant = !lean_ok ? 1 : ((int64_t)((M + 127) / 128) * ((N + 127) / 128) * splits <= 256 ? 3 : 2);
   if (variant != 1 && !lean_ok)
     BT_REFUSE("gemm_tile: this form needs K %d to be a multiple of 64 and operands below 4 GiB", K);
+  if (variant >= 4) return launch_deep(s, variant, a, lda, w, M, N, K, *epi, splits);
   int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
   dim3 grid(tiles_m * tiles_n, 1, splits);
   if (variant == 3) {

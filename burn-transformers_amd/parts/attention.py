@@ -101,7 +101,8 @@ class CausalSelfAttention(Mixer):
     def forward(self, h, step, memory, stream):
         tokens = h.shape[0]
         kv = memory.kv()
-        if memory.writes and tokens > 64 and step.dtype_is_bf16 and K.library_products():
+        if memory.writes and step.dtype_is_bf16 and not self.plain_only and \
+                K.prompt_products_in_library(tokens, self.n_q + 2 * self.n_kv, self.width, h.stride(0) if hasattr(h, "stride") else self.width):
             # a prompt: the vendor's library makes the whole projection, then keys and values are
             # copied into the cache; the queries are read where they lie
             qkv = step.buffer("attention.qkv", tokens, self.n_q + 2 * self.n_kv, step.dtype)

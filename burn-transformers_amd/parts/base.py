@@ -51,11 +51,15 @@ class ResidualStream:
     def add_product(self, step, a, weight, bias=None, packed=None):
         """x += a . weight^T + bias.  In a decode step (up to 64 rows) a product with few
         output columns splits its K range into partial sums that stay pending: the extra work-groups
-        are needed to pull the matrix through HBM.  Otherwise the product's epilogue adds into the
+        are needed to pull the matrix through HBM; so does a bfloat16 product of a short prompt or
+        chunk (``kernels.library.deep_split_count``).  Otherwise the product's epilogue adds into the
         stream in place.  ``packed``: the weight's ``kernels.library.PackedWeight``, if it has one."""
         rows, width = a.shape[0], weight.shape[0]
         if self.in_place:
             splits = 1
+        elif step.dtype_is_bf16 and rows > 64:       # a short prompt or chunk: the tile kernel's deep forms
+            splits = K.deep_split_count(rows, width, a.shape[1], compute_units(a.device)) \
+                if not isinstance(a, K.Chunked) and a.stride(1) == 1 and K.deep_form_rows(rows, a.shape[1], a.stride(0), width) else 1
         elif step.dtype_is_bf16:
             splits = split_count(rows, width, a.shape[1], compute_units(a.device), 32)
         elif a.shape[1] % 4 == 0 and a.stride(0) % 4 == 0:        # what the float32 MFMA kernels take

@@ -67,10 +67,11 @@ def test_gemm_epilogues(impl, dtype, m, n, k):
         assert float((out32.cpu().double() - want2).abs().max()) < 1e-5 * math.sqrt(k)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3])
-@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (300, 517, 1600), (130, 96, 192), (1000, 1600, 6400)])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (300, 517, 1600), (130, 96, 192), (1000, 1600, 6400), (65, 40, 128)])
 def test_tile_gemm_forms_agree(variant, m, n, k):
-    """The three forms of the tile kernel (any K; lean; direct to LDS) against float64."""
+    """The forms of the tile kernel (any K; lean; direct to LDS; direct to LDS with tiles of 64 x 64
+    and of 128 x 64 in more stages than K has tiles, or fewer) against float64."""
     a, w, bias, want = operands(m, n, k, torch.bfloat16, seed=variant, lda=k + 64)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
     K.gemm(a, w, K.epilogue_act(out, "gelu_erf", bias), impl="tile", variant=variant)

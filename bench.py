@@ -204,13 +204,19 @@ def kernel_classes(engine, entries, attention_bytes, attention_flops, peak_flops
     if not engine.use_programs:
         return {}
     graphs, engine.use_graphs = engine.use_graphs, False
+    before = [engine.length(slot) for slot, _ in entries]
     try:
-        engine.step(entries)
-        torch.cuda.synchronize()
+        for attempt in range(3):     # a step that made a workspace grow leaves no list: it is rewound and run again
+            engine.step(entries)
+            torch.cuda.synchronize()
+            if engine.last_program is not None:
+                break
+            for (slot, _), length in zip(entries, before):
+                engine.truncate(slot, length)
     finally:
         engine.use_graphs = graphs
     program = engine.last_program
-    if program is None:          # the step made a workspace grow, and a list recorded meanwhile is not kept
+    if program is None:
         return {}
     classes = {}
     for lib, name, call in program.calls:

@@ -98,10 +98,13 @@ class Chunked:
     stands where a tensor [rows, columns] would; whoever only hands it on to ``gemm``, ``add_norm``
     or ``attention_args`` needs to know nothing of it."""
 
-    # Steps of 17 to 64 rows use it.  Up to 16 rows it loses: the norm's rows are written by one
+    # Steps of 9 to 64 rows use it.  Up to 8 rows it loses: the norm's rows are written by one
     # work-group each, and two rows share every 128-byte line of a chunk (measured at 8 rows: the
     # norm 4.0 -> 4.6 us, the products behind it 6.3 -> 6.8 us; at 64 rows a step gains 5 %).
-    MIN_ROWS, MAX_ROWS = 17, 64
+    # Measured as ms a decode step, row-major / chunk-major, at three widths (12 layers of width 768,
+    # 24 of 1,024, 12 of 1,600): 12 rows 0.413 / 0.406, 0.837 / 0.823, 0.619 / 0.611; 16 rows
+    # 0.433 / 0.423, 0.908 / 0.888, 0.654 / 0.638.
+    MIN_ROWS, MAX_ROWS = 9, 64
     enabled = True        # tests switch it off to compare with row-major activations
 
     @classmethod
@@ -138,11 +141,13 @@ class Normalized:
     bfloat16 products, width up to 2048), which saves the norm's own kernel in front of it."""
 
     MAX_ROWS, MAX_WIDTH = 16, 2048          # what the kernel takes
-    # what pays: from nine rows on a wave normalises two rows one after the other, and the norm as
-    # a kernel of its own in front of an ordinary product is faster again.  Measured at GPT-2 XL's
-    # layer sizes, ms a decode step of 12 layers with the norm folded up to 16 rows / up to 8 rows:
-    # 0.586 / 0.571 at batch 9, 0.666 / 0.651 at batch 12, 0.724 / 0.681 at batch 16.
-    WORTH_ROWS = 8
+    # What pays: every work-group normalises all rows, a wave one row after the other from nine rows
+    # on, so the fold is worth it while a wave has at most this many elements to normalise; beyond,
+    # the norm as a kernel of its own in front of an ordinary product is faster again.  Measured as
+    # ms a decode step with the norm folded up to 8 rows / up to 16 rows: width 768 (12 layers) 0.425 /
+    # 0.413 at batch 12 and 0.438 / 0.433 at 16; width 1,024 (24 layers) 0.847 / 0.837 and 0.908 / 0.908;
+    # width 1,600 (12 layers) 0.651 / 0.666 at batch 12 and 0.681 / 0.724 at 16.
+    WORTH_ELEMENTS = 2048
 
     def __init__(self, x, gamma, beta, eps, kind):
         self.x, self.gamma, self.beta, self.eps, self.kind = x, gamma, beta, eps, kind
@@ -158,7 +163,7 @@ class Normalized:
     @classmethod
     def worth_it(cls, rows, width):
         """Whether a norm in front of a product should be folded into it."""
-        return rows <= cls.WORTH_ROWS and cls.possible(rows, width)
+        return cls.possible(rows, width) and (rows + 7) // 8 * width <= cls.WORTH_ELEMENTS
 
 
 # Every kernel of a step is called through its structure form, bt_<kernel>_call(stream, structure)

@@ -234,6 +234,15 @@ def packed_for_stream(weight):
     return K.PackedWeight(weight, (splits, 1))       # (without a split where the norm behind it is folded)
 
 
+# What a slice costs beyond the product itself, in the units of ``split_count`` (a work-group's time
+# for one chunk of K): the norm behind the product reads every slice's partial sums.  Measured as ms
+# a decode step with 0 / 1 / 2 / 3 (12 layers of width 768, 24 of width 1,024, 12 of width 1,600): 24
+# rows 0.512 / 0.506 / 0.501 / 0.498, 1.061 / 1.039 / 1.047 / 1.055 and 0.756 / 0.755 / 0.758 / 0.755; 64
+# rows 0.707 / 0.699 / 0.695 / 0.694, 1.598 / 1.566 / 1.585 / 1.598 and 1.198 / 1.196 / 1.199 / 1.197 (at
+# width 1,024 a step of 17 rows cut K = 1,024 into eight slices of four chunks without it).
+SPLIT_READ_COST = 1
+
+
 def split_count(rows, columns, k, units=256, chunk=32):
     """How many ways a residual-writing product splits its K range (up to 64 rows; 1 beyond).
 
@@ -254,7 +263,7 @@ def split_count(rows, columns, k, units=256, chunk=32):
         if splits > 1 and (per < 4 or per * (splits - 1) >= chunks):    # slices too thin, or an empty one
             continue
         rounds = (tiles * splits + units - 1) // units
-        cost = rounds * (per + 10)
+        cost = rounds * (per + 10) + SPLIT_READ_COST * splits
         if best_cost is None or cost < best_cost:
             best, best_cost = splits, cost
     return best

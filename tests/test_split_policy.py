@@ -35,6 +35,19 @@ def test_choices_at_measured_sizes():
     assert split_count(8, 50257, 1600) == 1
     # beyond 16 rows a work-group owns 32 columns, so there are half as many tiles to spread
     assert split_count(64, 1600, 6400) >= split_count(8, 1600, 6400)
+    # every slice is read again by the norm behind the product: K = 1,024 is not cut into eight slices of
+    # four chunks where four of eight do nearly as well (a step of 17 rows at width 1,024 was 2 % slower)
+    assert split_count(17, 1024, 1024) == 4
+
+
+def test_a_folded_norm_is_worth_it_by_rows_and_width():
+    """Up to eight rows at every width the kernel takes; nine to sixteen rows only where a wave's two
+    rows are short (measured at widths 768, 1,024 and 1,600)."""
+    from burn_transformers_amd.kernels.library import Normalized
+    assert all(Normalized.worth_it(8, width) for width in (768, 1024, 1600, 2048))
+    assert Normalized.worth_it(16, 768) and Normalized.worth_it(9, 1024) and Normalized.worth_it(16, 1024)
+    assert not Normalized.worth_it(9, 1600) and not Normalized.worth_it(16, 1280)
+    assert not Normalized.worth_it(17, 768) and not Normalized.worth_it(4, 4096) and not Normalized.worth_it(4, 772)
 
 
 # --- the runs a decode step's keys are cut into, and the classes of context ---------------------

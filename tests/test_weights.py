@@ -239,7 +239,7 @@ def test_chunk_major_layout_of_activations():
                 flat[((c // chunk) * rows + r) * chunk + c % chunk] = want[r, c]
         assert torch.equal(held.to_rows(), want)
         assert held.stride(0) == columns and held.stride(1) == 1 and held.dtype == dtype
-    assert [Chunked.wanted(n) for n in (1, 16, 17, 64, 65)] == [False, False, True, True, False]
+    assert [Chunked.wanted(n) for n in (1, 8, 9, 64, 65)] == [False, False, True, True, False]
     Chunked.enabled = False
     try:
         assert not Chunked.wanted(32)

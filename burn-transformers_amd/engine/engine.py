@@ -31,6 +31,7 @@ import time
 import numpy as np
 import torch
 
+from ..cache.ledger import BLOCK
 from ..cache.storage import Cache
 from ..kernels import library as K
 from .step import BufferPool, Step, StepLayout, StepPlan
@@ -75,6 +76,7 @@ class Engine:
         self._programs = {}                # shape -> (Program, logits), in order of last use
         self._programs_generation = -1     # the workspace generation the lists were recorded for
         self.program_runs = 0
+        self.programs_recorded = 0         # steps that ran from the parts and left a launch list
         self.last_program = None           # the launch list of the latest step, if it ran from one or left one
         self._meta = None                  # device int32 buffer of eager steps
         self._pinned = []                  # ring of (pinned int32 tensor, event)
@@ -268,46 +270,69 @@ class Engine:
         return self.model.forward(step, self.cache)
 
     def _run_program(self, plan, readout):
-        """The step from its launch list.  The first time a shape comes the parts run as always and
-        launch as they go (the GPU starts at once), and every kernel call is kept as well; from
-        then on the list is walked in C++.  A list names workspaces by address, so a workspace that
-        had to grow makes all lists stale, and a list recorded while one grew is not kept."""
+        """The step from its launch list.  The first time a class of steps comes (``token_capacity``:
+        a step of up to 64 tokens is a class of its own) the parts run as always and launch as they
+        go (the GPU starts at once), and every kernel call is kept as well; from then on the list is
+        walked in C++, for any step of the class: the counts in its calls are set to the step's
+        (``Program.set_shape``), everything else in them (addresses of weights, workspaces and
+        tables, pitches, kernels chosen) is the same for the whole class.  A list names workspaces
+        by address, so a workspace that had to grow makes all lists stale, and a list recorded while
+        one grew is not kept."""
         if self._programs_generation != self.pool.generation:
             self._programs.clear()
             self._programs_generation = self.pool.generation
             # (measurements under way were of lists that are gone; decisions taken stay)
             self._launch_bound = {k: v for k, v in self._launch_bound.items() if isinstance(v, bool)}
-        key = (plan.layout.key(), plan.max_count, readout, plan.context_limit if plan.decode else 0)
+        layout = plan.layout
+        exact = (layout.key(), plan.max_count, readout, plan.context_limit if plan.decode else 0)
+        # a step of more than 64 tokens that is not one of single tokens shares its list with its class
+        shared = (layout.class_key(), readout) if layout.tokens > BLOCK and plan.max_count > 1 else None
+        key = shared if shared is not None and shared in self._programs else exact
         held = self._programs.pop(key, None)
-        if held is None:
-            step = Step(plan.layout, self._meta, self.pool, self.dtype, plan)
-            generation = self.pool.generation
-            program = K.Program()
-            with program.recording(launch=True):
-                logits = self.model.forward(step, self.cache, readout=readout)
-            if not readout:
-                logits = torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
-            self.last_program = None
-            if self.pool.generation != generation:
-                # A workspace grew while the step ran.  The launches themselves were in order and are
-                # right, but calls recorded before the growth name the old address, and so do all
-                # older lists: none is kept, and the shape records again when it next comes (the
-                # workspaces are then large enough from the start).
-                self._programs.clear()
-                self._programs_generation = self.pool.generation
-                return logits
-            while len(self._programs) >= _MAX_PROGRAMS:
-                self._programs.pop(next(iter(self._programs)))
-            self._programs[key] = (program, logits)
+        if held is not None:
+            program, logits = held
+            if program.patches is not None:
+                program.set_shape(layout.tokens, plan.max_count)
+            self._programs[key] = held                    # (again) the most recently used
             self.last_program = program
+            began = time.perf_counter()
+            try:
+                program.run()
+            except K.KernelError:
+                if program.patches is None:
+                    raise
+                # a kernel refused the counts of this step of the class (the vendor's library has no
+                # algorithm for its rows, say): the list is dropped and the step runs from the parts
+                self._programs.pop(key, None)
+                return self._run_program(plan, readout)
+            self._walk_seconds = time.perf_counter() - began
+            self.program_runs += 1
             return logits
-        self._programs[key] = held                        # (again) the most recently used
-        self.last_program = held[0]
-        began = time.perf_counter()
-        held[0].run()
-        self._walk_seconds = time.perf_counter() - began
-        self.program_runs += 1
-        return held[1]
+        step = Step(layout, self._meta, self.pool, self.dtype, plan)
+        generation = self.pool.generation
+        program = K.Program()
+        with program.recording(launch=True):
+            logits = self.model.forward(step, self.cache, readout=readout)
+        if not readout:
+            logits = torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        self.last_program = None
+        self.programs_recorded += 1
+        if self.pool.generation != generation:
+            # A workspace grew while the step ran.  The launches themselves were in order and are
+            # right, but calls recorded before the growth name the old address, and so do all
+            # older lists: none is kept, and the shape records again when it next comes (the
+            # workspaces are then large enough from the start).
+            self._programs.clear()
+            self._programs_generation = self.pool.generation
+            return logits
+        key = exact
+        if shared is not None and program.for_any_step_of_its_class(layout.tokens, plan.max_count, layout.rows):
+            key = shared
+        while len(self._programs) >= _MAX_PROGRAMS:
+            self._programs.pop(next(iter(self._programs)))
+        self._programs[key] = (program, logits)
+        self.last_program = program
+        return logits
 
     def _run_from_graph(self, plan, readout):
         # (parts plan decode steps by the class of context; steps with prompt tokens look the same in every class)
@@ -355,7 +380,8 @@ class Engine:
             if len(self._launch_bound) > 4096:
                 self._launch_bound.clear()
             probe = self._launch_bound[key] = []
-        if key not in self._programs and self._seen.get(key, 0) < 8:
+        shared = (plan.layout.class_key(), readout)
+        if key not in self._programs and shared not in self._programs and self._seen.get(key, 0) < 8:
             # the shape has no list (its first step made a workspace grow, or the lists were dropped
             # since): this step would be launched from Python and say nothing about the list; it
             # records, the next one is measured

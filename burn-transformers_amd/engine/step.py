@@ -20,22 +20,39 @@ def _align(n):
     return (n + 3) & ~3
 
 
+def token_capacity(tokens):
+    """The class of a step by its tokens: steps of up to 64 tokens are their own class; beyond, the
+    classes are 65 .. 128, 129 .. 192 and so on.  Every step of a class lays its tables out for the
+    class's most tokens and reserves its workspaces for them, and every choice of kernels that the
+    parts make by a step's rows is the same for a whole class (they turn at 64, 128 and 256 rows), so
+    that one launch list serves the class: only the counts in its calls differ from step to step."""
+    return tokens if tokens <= BLOCK else (tokens + BLOCK - 1) // BLOCK * BLOCK
+
+
 class StepLayout:
-    """Offsets of the sections for T tokens, B sequences, R wanted rows."""
+    """Offsets of the sections for T tokens, B sequences, R wanted rows.  The sections that hold one
+    word per token have room for the step's class (``token_capacity``), so that the later sections
+    start at the same place in every step of a class."""
 
     def __init__(self, tokens, seqs, rows, max_blocks, groups=1):
         self.tokens, self.seqs, self.rows, self.max_blocks, self.groups = tokens, seqs, rows, max_blocks, groups
+        self.capacity = token_capacity(tokens)
         offset = 0
         self.sections = {}
-        for name, size in (("tok_ids", tokens), ("tok_pos", tokens), ("tok_seq", tokens),
-                           ("seq_off", seqs + 1), ("seq_start", seqs), ("slots", seqs),
-                           ("sel_rows", rows), ("block_table", groups * seqs * max_blocks)):
+        for name, size, room in (("tok_ids", tokens, self.capacity), ("tok_pos", tokens, self.capacity),
+                                 ("tok_seq", tokens, self.capacity),
+                                 ("seq_off", seqs + 1, seqs + 1), ("seq_start", seqs, seqs), ("slots", seqs, seqs),
+                                 ("sel_rows", rows, rows), ("block_table", groups * seqs * max_blocks, groups * seqs * max_blocks)):
             self.sections[name] = (offset, size)
-            offset = _align(offset + size)
+            offset = _align(offset + room)
         self.total = offset
 
     def key(self):
         return (self.tokens, self.seqs, self.rows, self.max_blocks, self.groups)
+
+    def class_key(self):
+        """What the steps that one launch list serves have in common."""
+        return (self.capacity, self.seqs, self.rows, self.max_blocks, self.groups)
 
 
 class StepPlan:
@@ -96,6 +113,7 @@ class Step:
     def __init__(self, plan_or_layout, device_meta, pool, dtype, host_plan=None):
         layout = plan_or_layout
         self.n_tokens, self.n_seqs, self.max_blocks = layout.tokens, layout.seqs, layout.max_blocks
+        self.token_capacity = layout.capacity        # most tokens of a step of this class: workspaces are reserved for them
         for name, (offset, size) in layout.sections.items():
             setattr(self, name, device_meta[offset:offset + size])
         if self.n_seqs:       # [groups, sequences, blocks]; a mixer gets its group's table with its view of the cache
@@ -110,7 +128,19 @@ class Step:
         self.host = host_plan
 
     def buffer(self, key, rows, cols, dtype):
-        return self.pool.take(key, rows, cols, dtype)
+        """A workspace [rows, cols] that keeps its address from step to step.  One that holds a row
+        (or several) per token of the step is reserved for the most tokens of the step's class, so
+        that it stays where it is for every step of the class."""
+        reserve = rows
+        if self.n_tokens and self.token_capacity != self.n_tokens and rows % self.n_tokens == 0:
+            reserve = rows // self.n_tokens * self.token_capacity
+        return self.pool.take(key, rows, cols, dtype, reserve)
+
+    def partial_sums(self, key, splits, rows, cols):
+        """float32 [splits, rows, cols] for the slices of a product whose K range is cut, the slices
+        as far apart as the step's class needs: the same distance in every step of the class."""
+        room = self.token_capacity if rows == self.n_tokens else rows
+        return self.buffer(key, splits * room, cols, "float32").view(splits, room, cols)[:, :rows]
 
 
 class BufferPool:
@@ -121,7 +151,8 @@ class BufferPool:
         self.device, self.buffers, self.generation, self.frozen = device, {}, 0, False
         self.views = {}         # (key, dtype, rows, cols) -> the view handed out last time: a step asks hundreds of times
 
-    def take(self, key, rows, cols, dtype):
+    def take(self, key, rows, cols, dtype, reserve_rows=0):
+        """``reserve_rows``: rows to make room for where the workspace has to be made or replaced."""
         view = self.views.get((key, dtype, rows, cols))
         if view is not None:
             return view
@@ -131,6 +162,7 @@ class BufferPool:
         need = rows * cols
         held = self.buffers.get((key, dtype))
         if held is None or held.numel() < need:
+            need = max(need, reserve_rows * cols)
             if self.frozen:
                 raise RuntimeError(f"workspace {key!r} would have to grow while a graph is being captured")
             if held is not None:
@@ -138,7 +170,7 @@ class BufferPool:
                 self.views = {k: v for k, v in self.views.items() if k[0] != key}      # they show the old memory
             held = torch.empty(max(need, 1), dtype=dtype, device=self.device)
             self.buffers[(key, dtype)] = held
-        view = held[:need].view(rows, cols)
+        view = held[:rows * cols].view(rows, cols)
         if len(self.views) > 4096:
             self.views.clear()
         self.views[(key, asked, rows, cols)] = view

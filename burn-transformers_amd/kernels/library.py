@@ -232,6 +232,33 @@ def _launch(lib, name, call):
     _check(lib, getattr(lib, name)(_stream(), ctypes.byref(call)))
 
 
+# The fields of the call structures that hold a step's number of tokens ("tokens") or the most tokens
+# one of its sequences brings ("max_count"): what differs between the launch lists of two steps of
+# one class (``engine.step.token_capacity``).  A part that brings a kernel of its own says the same of
+# its structure with a class attribute ``_step_fields_ = {"field": "tokens"}``; a structure that says
+# nothing keeps a list from serving any step but the one it was recorded for.
+def _step_fields(call):
+    kind = type(call)
+    if kind is GemmCall:
+        return (("M", "tokens"),)
+    if kind is AddNormCall:
+        return () if call.rows else (("n_rows", "tokens"),)        # (with a selection of rows: the wanted rows)
+    if kind is EmbedCall or kind is KvCopyCall:
+        return (("tokens", "tokens"),)
+    if kind is AttentionCall:
+        return (("args.n_tokens", "tokens"), ("args.max_count", "max_count"))
+    declared = getattr(kind, "_step_fields_", None)
+    return None if declared is None else tuple(declared.items())
+
+
+def _field(call, path):
+    """(the structure that holds the field, its name) of a dotted path."""
+    *outer, name = path.split(".")
+    for part in outer:
+        call = getattr(call, part)
+    return call, name
+
+
 class Program:
     """A launch list: the kernel calls of one step, in order, each as (entry point, argument
     structure).  ``run`` hands the whole list to one C++ loop (csrc/program.cpp), so a step costs
@@ -253,6 +280,43 @@ class Program:
         self.calls = []             # (module, entry point name, structure); the structures are kept alive here
         self._entries = None
         self.launch_while_recording = False
+        self.patches = None         # see ``for_any_step_of_its_class``
+        self.shape = None           # (tokens, max_count) the structures hold now
+
+    def for_any_step_of_its_class(self, tokens, max_count, wanted_rows):
+        """Finds the fields of the list's calls that hold the step's counts, so that the list can
+        be run for another step of the same class (``set_shape``).  ``tokens``, ``max_count`` and
+        ``wanted_rows`` are those of the step it was recorded for.  Returns False, and leaves the
+        list good for steps of exactly that shape only, if a call does not say which of its fields
+        they are, or holds a row count that is neither the step's tokens nor its wanted rows (or
+        could be either)."""
+        patches = []
+        for _, _, call in self.calls:
+            fields = _step_fields(call)
+            if fields is None:
+                return False
+            for path, what in fields:
+                holder, name = _field(call, path)
+                value = getattr(holder, name)
+                if what == "max_count":
+                    if value != max_count:
+                        return False
+                elif value == tokens and tokens != wanted_rows:
+                    pass
+                elif value == wanted_rows and tokens != wanted_rows and type(call) is GemmCall:
+                    continue                   # the readout's product: its rows are the wanted ones
+                else:
+                    return False
+                patches.append((holder, name, what))
+        self.patches, self.shape = patches, (tokens, max_count)
+        return True
+
+    def set_shape(self, tokens, max_count):
+        """Makes the list that of a step of ``tokens`` tokens, ``max_count`` at most of one sequence."""
+        if self.shape != (tokens, max_count):
+            for holder, name, what in self.patches:
+                setattr(holder, name, tokens if what == "tokens" else max_count)
+            self.shape = (tokens, max_count)
 
     def add(self, lib, name, call):
         self.calls.append((lib, name, call))

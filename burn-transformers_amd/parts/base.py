@@ -67,7 +67,7 @@ class ResidualStream:
         else:
             splits = 1
         if splits > 1:
-            partials = step.buffer("stream.partials", splits * rows, width, "float32").view(splits, rows, width)
+            partials = step.partial_sums("stream.partials", splits, rows, width)
             K.gemm(a, weight, K.epilogue_f32(partials), splits=splits, packed=packed)
             self.add(Delta(partials, bias))
         else:

@@ -53,8 +53,9 @@ def test_steps_from_launch_lists_equal_steps_issued_one_by_one(name, dtype):
         shapes.add(tuple(len(e[1]) for e in entries_l))
         for i, e in zip(chosen, entries_l):
             fed[i] += len(e[1])
-    # a shape's first step launches as it records; every later one runs from its list
-    assert listed.program_runs < listed.steps_run and len(listed._programs) > 0 and direct.program_runs == 0
+    # a shape's first step launches as it records; every later one runs from its list (the lists kept
+    # now may be none: a workspace that grows in the last step drops them all)
+    assert 0 < listed.program_runs < listed.steps_run and direct.program_runs == 0
     # and against the plain implementation, through the list that was used most recently
     ids = requests[1]
     slot = listed.open()
@@ -163,3 +164,68 @@ def test_the_engine_chooses_a_path_for_a_repeating_shape_by_itself():
     assert (engine.graph_replays > 0) == (decisions[0] is False)
     want = plain_logits("A", ids)
     assert float((torch.cat(rows).cpu().double() - want).abs().max()) <= tolerance("bfloat16", want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "BW"])
+def test_one_launch_list_serves_every_prompt_length_of_its_class(name, dtype):
+    """Prompts of 65 to 128 tokens (and 129 to 190), in random order, on an engine that walks launch
+    lists and on one that issues every kernel from Python: the same bits, and the first engine has
+    recorded ONE list for each class of lengths (65 .. 128, 129 .. 192), whose counts it sets to
+    each step's; a step with other wanted rows, or of several sequences, is another class."""
+    model = model_for(name, dtype)
+    listed = bt.Engine(model, max_tokens=64 * 8, graphs=False)
+    direct = bt.Engine(model, max_tokens=64 * 8, graphs=False, programs=False)
+    gen = torch.Generator().manual_seed(17)
+    limit = model.max_positions
+    lengths = [65, 128, 70, 127, 100, 66, 96] + torch.randint(65, 129, (8,), generator=gen).tolist()
+    if limit >= 190:
+        lengths += [129, 190, 150, 64, 65]
+    lengths = [n for n in lengths if n < limit]            # (one more token follows every prompt)
+    classes = {n if n <= 64 else (n + 63) // 64 for n in lengths}
+
+    def walk(order):
+        for n in order:
+            ids = prompts_for(name, [n], seed=1000 + n)[0]
+            a, b = listed.open(), direct.open()
+            got, want = listed.step([(a, ids)]).clone(), direct.step([(b, ids)])
+            assert torch.equal(got, want), f"a prompt of {n} tokens"
+            # the cache holds the same too: one more token on both gives the same bits
+            got, want = listed.step([(a, [ids[0]])]).clone(), direct.step([(b, [ids[0]])])
+            assert torch.equal(got, want), f"the token after a prompt of {n} tokens"
+            listed.close(a)
+            direct.close(b)
+        return ids
+
+    # One prompt of every class, the longest first, twice over: the workspaces then have their sizes
+    # (a list recorded while one grew is not kept, and growth drops the older lists) and every class
+    # has its list.  From then on no step of any of these lengths is issued from Python again.
+    firsts = sorted({max(n for n in lengths if (n if n <= 64 else (n + 63) // 64) == c) for c in classes}, reverse=True)
+    walk(firsts + firsts)
+    recorded, runs, steps = listed.programs_recorded, listed.program_runs, listed.steps_run
+    ids = walk(lengths)
+    assert listed.programs_recorded == recorded, f"{listed.programs_recorded - recorded} steps were issued from Python again"
+    assert listed.program_runs - runs == listed.steps_run - steps == 2 * len(lengths)
+    assert len(listed._programs) == len(classes) + 1           # one list a class, and the step of one token
+    assert direct.program_runs == 0
+    # the last prompt against the plain implementation: the lists are not only equal to the direct path
+    reference = plain_logits(name, ids)[-1:]
+    logits = listed.step([(listed.open(), ids)])
+    assert float((logits.cpu().double() - reference).abs().max()) <= tolerance(dtype, reference)
+    # two sequences of unequal lengths, all rows wanted for one of them: classes of their own
+    first, second = prompts_for(name, [70, 30], seed=5)
+    for _ in range(2):
+        a, b = (listed.open(), listed.open()), (direct.open(), direct.open())
+        for cut in ((40, 30), (30, 0)):
+            entries = [(first[:40] if cut[0] == 40 else first[40:]), (second if cut[1] else [])]
+            want_rows = [list(range(len(entries[0]))), []]
+            got = listed.step(list(zip(a, entries)), want=want_rows).clone()
+            want = direct.step(list(zip(b, entries)), want=want_rows)
+            assert torch.equal(got, want)
+        for slot in a:
+            listed.close(slot)
+        for slot in b:
+            direct.close(slot)
+    listed.reset()
+    direct.reset()
+    listed.cache.ledger.check()

@@ -227,17 +227,20 @@ def test_blocks_with_other_roles_no_mixer_and_a_turning_mixer(dtype, tmp_path):
         listed = bt.Engine(model, max_tokens=1024, graphs=False)
         direct = bt.Engine(model, max_tokens=1024, graphs=False, programs=False)
         assert listed.use_programs and not direct.use_programs
-        for round_ in range(2):                 # the second round's shapes are walked from their lists
+        for round_ in range(3):                 # the last round's steps are all walked from their lists
+            runs_before = listed.program_runs
             pairs = [(listed.open(), direct.open()) for _ in requests]
             for begin, end in ((0, 5), (5, 6), (6, 7), (7, 9)):
                 a = listed.step([(p[0], r[begin:end]) for p, r in zip(pairs, requests)]).clone()
                 b = direct.step([(p[1], r[begin:end]) for p, r in zip(pairs, requests)]).clone()
                 assert torch.equal(a, b), f"round {round_} tokens {begin}..{end}"
-            assert any(name == "bt_toy_rotary_turn_call" for _, name, _ in listed.last_program.calls)
+            if round_ == 2:            # (earlier steps may have made workspaces grow, which drops the lists kept till then)
+                assert any(name == "bt_toy_rotary_turn_call" for _, name, _ in listed.last_program.calls)
+                assert listed.program_runs - runs_before == 4
             for a, b in pairs:
                 listed.close(a)
                 direct.close(b)
-        assert listed.program_runs >= 5 and direct.program_runs == 0
+        assert direct.program_runs == 0
     finally:
         unregister("block", "toy_side_by_side")
         unregister("block", "toy_channels_only")

@@ -13,6 +13,9 @@ class RotaryTurnCall(ctypes.Structure):
     _fields_ = [("dtype", ctypes.c_int), ("tokens", ctypes.c_int), ("parts", ctypes.c_int), ("heads", ctypes.c_int),
                 ("head_dim", ctypes.c_int), ("ld", ctypes.c_int64), ("rows", ctypes.c_void_p),
                 ("positions", ctypes.c_void_p), ("freq", ctypes.c_void_p)]
+    # the field that holds a step's number of tokens: with it said, a launch list that holds such a
+    # call serves every step of its class, not only the one it was recorded for
+    _step_fields_ = {"tokens": "tokens"}
 
 
 def register():

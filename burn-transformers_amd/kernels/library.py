@@ -657,11 +657,11 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
             impl = "skinny"
         elif dtype == FLOAT32:
             impl = "tile"
-        elif deep_form_rows(m, k, a.stride(0), n):
+        elif deep_form_rows(m, k, a.stride(0), n, sliced=splits > 1):
             # short prompts and chunks: the tile kernel's deep forms (see ``deep_form_rows``)
             impl = "tile"
-            if variant == 0:     # tiles of 64 x 64 (eight stages where K is cut into slices), of 128 x 64 beyond 128 rows
-                variant = (4 if splits > 1 else 5) if m <= 128 or splits > 1 else 7
+            if variant == 0:     # tiles of 64 x 64 in four stages; of 128 x 64 beyond 128 rows where K is whole
+                variant = 5 if m <= 128 or splits > 1 else 7
         else:
             impl = "library" if splits == 1 and _library_takes(epilogue) and library_products() \
                 and _library_has_algorithm(a.stride(0), m, n, k, epilogue) else "tile"
@@ -689,30 +689,39 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
         _launch(_module("gemm_mfma"), "bt_gemm_skinny_call", call)
 
 
-DEEP_FORM_ROWS = 256       # most rows of a bfloat16 product that the tile kernel's deep forms take
+DEEP_FORM_ROWS = 256          # most rows of a bfloat16 product that the tile kernel's deep forms take ...
+DEEP_FORM_SLICED_ROWS = 512   # ... and of one that leaves partial sums of slices of K pending
 
 
-def deep_form_rows(m, k, lda, n):
+def deep_form_rows(m, k, lda, n, sliced=False):
     """Whether a bfloat16 product of ``m`` rows is one for the tile kernel's deep forms (tiles of
-    64 x 64 or 128 x 64 brought straight into LDS, up to seven of them on their way at once): 65 to
+    64 x 64 or 128 x 64 brought straight into LDS, several of them on their way at once): 65 to
     256 rows, where it has too few tiles of 128 x 128 to fill the chip and the vendor's library
     takes 16 to 24 us whatever the shape (measured at widths 1,600 and 6,400: these forms take a
-    quarter to a third less, and up to 45 % less where K is cut into slices of pending partial
-    sums); from 512 rows on the library wins.  The forms read K in tiles of 64 and address their
-    operands with 32 bits."""
-    return 64 < m <= DEEP_FORM_ROWS and k % 64 == 0 and m * lda * 2 < (1 << 32) and n * k * 2 < (1 << 32)
+    quarter to a third less); where the product may leave slices of K pending (``sliced``: the two
+    products that add to the residual stream) up to 512 rows, and up to 45 % less.  Beyond, the
+    library wins.  The forms read K in tiles of 64 and address their operands with 32 bits."""
+    limit = DEEP_FORM_SLICED_ROWS if sliced else DEEP_FORM_ROWS
+    return 64 < m <= limit and k % 64 == 0 and m * lda * 2 < (1 << 32) and n * k * 2 < (1 << 32)
 
 
 def deep_split_count(rows, columns, k, units=256):
     """Into how many slices of pending partial sums a residual-writing bfloat16 product of 65 to
-    ``DEEP_FORM_ROWS`` rows cuts its K range: as many as give every compute unit a tile of 64 x 64,
-    at most four (the norm behind it reads them all), each at least four tiles of K long.
-    Measured at width 1,600 (us, slices 1 / 2 / 4): 128 rows 1600 x 1600 12.2 / 8.1 / 6.7 and 1600 x
-    6400 34.8 / 20.1 / 13.4; 256 rows 12.4 / 8.4 / 11.4 and 34.5 / 20.6 / 23.8."""
-    if not deep_form_rows(rows, k, k, columns):
+    ``DEEP_FORM_SLICED_ROWS`` rows cuts its K range: as many as still give every work-group (a tile
+    of 64 x 64 of one slice) a compute unit of its own, or, where even two slices are too many for
+    that, as many as leave at most two work-groups to a unit; at most four (the norm behind the
+    product reads them all), each at least four tiles of K long.  Measured at width 1,600 on 256
+    units (us for 1600 x 1600 and 1600 x 6400, slices 2 / 3 / 4): 128 rows 7.1 / 6.3 / 5.9 and 18.9 /
+    14.5 / 12.1; 192 rows 7.3 / 6.5 / 7.2 and 18.8 / 14.7 / 18.8; 256 rows 7.4 / 7.9 / 7.5 and 19.2 /
+    22.4 / 18.8; 384 rows 9.3 / 8.4 / 10.9 and 29.3 / 23.1 / 26.5; 512 rows 9.5 / 12.1 / 12.1 and 30.7 /
+    32.2 / 31.0 (the vendor's library: 11.1 to 12.2 and 18.3 to 32.4)."""
+    if not deep_form_rows(rows, k, k, columns, sliced=True):
         return 1
     tiles = ((rows + 63) // 64) * ((columns + 63) // 64)
-    return max(1, min(4, units // tiles, (k // 64) // 4))
+    splits = units // tiles
+    if splits < 2:
+        splits = 2 * units // tiles
+    return max(1, min(4, splits, (k // 64) // 4))
 
 
 def prompt_products_in_library(m, n, k, lda):

@@ -59,7 +59,8 @@ class ResidualStream:
             splits = 1
         elif step.dtype_is_bf16 and rows > 64:       # a short prompt or chunk: the tile kernel's deep forms
             splits = K.deep_split_count(rows, width, a.shape[1], compute_units(a.device)) \
-                if not isinstance(a, K.Chunked) and a.stride(1) == 1 and K.deep_form_rows(rows, a.shape[1], a.stride(0), width) else 1
+                if not isinstance(a, K.Chunked) and a.stride(1) == 1 and \
+                K.deep_form_rows(rows, a.shape[1], a.stride(0), width, sliced=True) else 1
         elif step.dtype_is_bf16:
             splits = split_count(rows, width, a.shape[1], compute_units(a.device), 32)
         elif a.shape[1] % 4 == 0 and a.stride(0) % 4 == 0:        # what the float32 MFMA kernels take

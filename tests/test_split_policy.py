@@ -105,20 +105,24 @@ def test_whether_a_graph_pays_is_decided_by_the_median_of_the_measured_steps():
 
 def test_products_of_short_prompts_and_how_they_cut_k():
     """``deep_form_rows`` / ``deep_split_count``: 65 to 256 rows with K a multiple of 64 go to the
-    tile kernel's deep forms; a residual-writing one cuts K so that every compute unit has a tile,
-    into at most four slices of at least four tiles of K."""
+    tile kernel's deep forms, up to 512 where slices of K may stay pending; a residual-writing one
+    cuts K so that every work-group has a compute unit, or at most two share one, into at most four
+    slices of at least four tiles of K."""
     from burn_transformers_amd.kernels.library import deep_form_rows, deep_split_count
     assert not deep_form_rows(64, 1600, 1600, 4800) and deep_form_rows(65, 1600, 1600, 4800)
     assert deep_form_rows(256, 1600, 1600, 4800) and not deep_form_rows(257, 1600, 1600, 4800)
+    assert deep_form_rows(512, 1600, 1600, 1600, sliced=True) and not deep_form_rows(513, 1600, 1600, 1600, sliced=True)
     assert not deep_form_rows(128, 1608, 1608, 4800)            # K in tiles of 64
     assert not deep_form_rows(128, 64, 1 << 25, 64)             # operands addressed with 32 bits
     assert deep_split_count(128, 1600, 1600) == 4 and deep_split_count(128, 1600, 6400) == 4
+    assert deep_split_count(192, 1600, 1600) == 3 and deep_split_count(192, 1600, 6400) == 3
     assert deep_split_count(256, 1600, 1600) == 2 and deep_split_count(256, 1600, 6400) == 2
+    assert deep_split_count(384, 1600, 6400) == 3 and deep_split_count(512, 1600, 6400) == 2     # two work-groups a unit
     assert deep_split_count(128, 768, 768) == 3                 # 12 tiles of K: three slices of four
     assert deep_split_count(100, 64, 64) == 1 and deep_split_count(100, 64, 256) == 1   # K too short to cut
-    assert deep_split_count(200, 6400, 1600) == 1               # tiles enough without a cut
-    assert deep_split_count(64, 1600, 1600) == 1 and deep_split_count(300, 1600, 1600) == 1
-    for rows in (65, 100, 128, 200, 256):
+    assert deep_split_count(512, 6400, 1600) == 1               # tiles enough without a cut
+    assert deep_split_count(64, 1600, 1600) == 1 and deep_split_count(513, 1600, 1600) == 1
+    for rows in (65, 100, 128, 200, 256, 300, 512):
         for columns in (64, 768, 1024, 1600, 50257):
             for k in (64, 128, 768, 1024, 1600, 6400):
                 splits = deep_split_count(rows, columns, k)

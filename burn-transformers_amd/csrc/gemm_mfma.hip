@@ -472,17 +472,25 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
 // chunks of prompts): a template over the tile (BM x BN, 64 or 128 each, four waves as 2 x 2) and
 // the number of stages.  Such a product has too few tiles of 128 x 128 to fill the chip, and with
 // smaller tiles a work-group has less arithmetic per byte it pulls, so that its time is the 25 (or
-// 100) trips to memory of its loop over K unless many of them are in flight at once: a tile of
-// 64 x 64 is 16 KiB a stage, and eight stages keep seven tiles (112 KiB) on their way while one is
-// multiplied.  Same layout of a stage as above (A's rows, then W's, 128 bytes each, the swizzle
-// applied on the memory side), same waits written by hand.  K a multiple of 64, operands below 4 GiB.
-// Measured at 128 rows (us; the vendor's library beside it): 4800 x 1600 12.0 (17.3), 6400 x 1600 13.6
-// (18.2), and with K cut into four slices of pending partial sums 1600 x 1600 6.7 (11.2), 1600 x 6400
-// 13.4 (18.4); at 256 rows tiles of 128 x 64 take 17.4 (20.0) and 20.0 (21.4), two slices of 64 x 64
-// 8.4 (11.7) and 20.6 (23.9); from 512 rows on the library wins.  What bounds these forms is their
-// loop of loads: with the matrix instructions and the LDS reads taken out the times stay (a
-// work-group gets a tile of 16 KiB every 0.4 us, whatever the number of stages), and a ring of
-// register sets in place of the direct loads was slower still.
+// 100) trips to memory of its loop over K unless several of them are in flight at once.  Same layout
+// of a stage as above (A's rows, then W's, 128 bytes each, the swizzle applied on the memory side),
+// same waits written by hand.  K a multiple of 64, operands below 4 GiB.
+// Measured at 128 rows (us; the vendor's library beside it): tiles of 64 x 64 in four stages 4800 x
+// 1600 12.0 (17.3), 6400 x 1600 13.6 (18.2), and with K cut into four slices of pending partial sums
+// 1600 x 1600 5.9 (11.2), 1600 x 6400 12.1 (18.4); at 256 rows tiles of 128 x 64 take 17.4 (20.0) and
+// 20.0 (21.4), two slices of 64 x 64 7.4 (11.7) and 19.2 (23.9); sliced products win up to 512 rows
+// (9.5 and 30.7 against 12.1 and 32.4), the others lose to the library from 512 rows on.  Four stages
+// (64 KiB, two work-groups to a compute unit) do as well as eight or better.
+// What bounds these forms is what the compute units pull, not what they multiply: a work-group
+// gets a tile of 64 x 64 (16 KiB) about every 0.4 us, one of 128 x 64 every 0.6 us and one of 128 x
+// 128 every 0.85 us, whatever the number of stages; with the matrix instructions and the LDS reads
+// taken out the times stay.  Measured and not taken, all at 128 rows and within 10 % of the above:
+// a ring of register sets in place of the direct loads (slower), waves that do nothing but issue the
+// loads (2, 4 or 8 loads a wave and tile: the same times), all rows of the step against 32 columns
+// with the weights in a ring of their own, 8 or 16 tiles deep, filled by a wave of its own (the
+// same), each work-group starting its walk over K at another tile (the same).  All work-groups
+// together pull at 6 to 12 TB/s through the L2s, more the more of them share a compute unit; a
+// kernel that only reads as much without a loop does 27 TB/s from the L2 and 6.6 from memory.
 template <int NEWER, int LOADS>
 __device__ __forceinline__ void wait_for_all_but(int newer) {
   // waits until at most `newer` tiles' loads (LOADS instructions each) of this wave are in flight

@@ -429,7 +429,7 @@ def run_sweep(args):
     print(f"# GPT-2 XL layer sizes, {layers} layers, 8,192 positions, {dtype}, random weights")
     print("# decode: one token per sequence from a HIP graph, every sequence holding `context` tokens")
     print("kind\tbatch\tcontext\tms_per_step\ttokens_per_s\thbm_fraction")
-    for context in (1024, 2048, 4096, 8192):
+    for context in (1024, 2048, 4096, 8192) if args.sweep_part in ("all", "decode") else ():
         for batch in (1, 8, 16, 32, 64):
             engine = bt.Engine(model, max_tokens=batch * (context + 64))
             slots = [engine.open() for _ in range(batch)]
@@ -454,7 +454,7 @@ def run_sweep(args):
     print("# prompts: one sequence, whole (chunk 0) or in chunks; the fraction is of the MFMA peak")
     print("kind\ttokens\tchunk\tms\ttokens_per_s\tmfma_fraction")
     engine = bt.Engine(model, max_tokens=8192 + 64)
-    for tokens in (64, 128, 256, 512, 1024, 2048, 4096, 8192):
+    for tokens in (64, 128, 256, 512, 1024, 2048, 4096, 8192) if args.sweep_part in ("all", "prompts") else ():
         for chunk in (0, 256):
             if chunk and tokens <= chunk:
                 continue
@@ -487,6 +487,8 @@ def main():
     parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
     parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
     parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep"], default="xl")
+    parser.add_argument("--sweep-part", choices=["all", "decode", "prompts"], default="all",
+                        help="which table of --workload sweep to run")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     parser.add_argument("--no-kernels", action="store_true", help="skip the classes of kernels on their own")
     parser.add_argument("--no-own", action="store_true", help="skip the prefill on this package's own product kernels")

@@ -19,9 +19,11 @@ struct AttnArgs {
   int max_count;        // most tokens any sequence brings in this step
   int window;           // 0 = all earlier keys
   float scale;
-  // Decode only: with splits > 1 the keys of every sequence are cut into that many runs, each run
-  // is a work-group of its own that leaves (output row, maximum, sum) in `partial`
-  // [n_seqs][q_heads][splits][head_dim + 2], and a second kernel joins them into `out`.
+  // With splits > 1 the keys are cut into that many runs, each run is a work-group of its own that
+  // leaves (output row, maximum, sum) in `partial` [rows][q_heads][splits][head_dim + 2], and a
+  // second kernel joins them into `out`.  Decode: the runs of every sequence's keys, a row is a
+  // sequence.  Prompts (bfloat16, heads of 64, no window): the runs of every query tile's keys, a
+  // row is a token of the step.
   int splits;
   float* partial;
   // Decode (bfloat16 MFMA kernels) only: 0, or `out` is chunk-major with that many rows

@@ -517,15 +517,22 @@ attention_prefill_split_kernel(AttnArgs a) {
   const int i16 = lane & 15, g = lane >> 4;
   // work-groups that read the same keys and values lie on one XCD (as in attention_prefill_kernel);
   // within an XCD the tiles come latest first, all (sequence, head) pairs of a rank together
+  // a.splits > 1: every tile's turns are cut into that many runs, a work-group each, which leave
+  // (unnormalised output row, maximum, sum) per query and head for attention_join_kernel: a chunk
+  // of a prompt behind a long context has few tiles of queries and many keys for each.  What
+  // shares keys is then a run of a (sequence, head) pair, and those are what is dealt to the XCDs
+  // (25 heads in 5 runs: 125 over 8, where whole pairs would give one XCD 4 x 5 and the others 3 x 5).
+  const int runs = a.splits > 1 ? a.splits : 1;
   const int group = a.q_heads / a.kv.kv_heads;
   const int q_tiles = (a.max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES;
-  const int units = a.n_seqs * a.kv.kv_heads, units_per_xcd = (units + 7) / 8;
+  const int units = a.n_seqs * a.kv.kv_heads * runs, units_per_xcd = (units + 7) / 8;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int per_rank = units_per_xcd * group;
   const int rank = slot / per_rank, inside = slot % per_rank;
   const int unit = (inside / group) * 8 + xcd;
   if (unit >= units) return;                                // the whole work-group
-  const int seq = unit / a.kv.kv_heads, kv_head = unit % a.kv.kv_heads;
+  const int pair = unit / runs, run = unit % runs;
+  const int seq = pair / a.kv.kv_heads, kv_head = pair % a.kv.kv_heads;
   const int head = kv_head * group + inside % group;
   const int q_tile = q_tiles - 1 - rank;
   const int off = a.seq_off[seq], count = a.seq_off[seq + 1] - off, start = a.seq_start[seq];
@@ -533,10 +540,15 @@ attention_prefill_split_kernel(AttnArgs a) {
   const int reach = (q_tile + 1) * PREFILL_QUERIES < count ? (q_tile + 1) * PREFILL_QUERIES : count;
   const int n_blocks = (start + reach + BT_KV_BLOCK - 1) / BT_KV_BLOCK;
   const int n_turns = (n_blocks + 1) / 2;
+  const int per_run = (n_turns + runs - 1) / runs;
+  const int t_begin = run * per_run;
+  const int t_end = t_begin + per_run < n_turns ? t_begin + per_run : n_turns;
+  const bool empty_run = t_begin >= t_end;                  // (the same for the whole work-group)
   // Every wave meets the others at the same barriers: one when the first turn is in place, one at
   // the end of every turn, one before the second set's results are read.
 
   if (brings) {
+    if (empty_run) return;
     const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
     const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
     typedef __attribute__((__vector_size__(2 * sizeof(int)))) int int2v;
@@ -574,14 +586,14 @@ attention_prefill_split_kernel(AttnArgs a) {
         }
       }
     };
-    fetch(0);
+    fetch(t_begin);
     stash(split_lds);
-    if (n_turns > 1) fetch(1);
+    if (t_begin + 1 < t_end) fetch(t_begin + 1);
     __syncthreads();                                         // the first turn is in place
-    for (int t = 0; t < n_turns; ++t) {
+    for (int t = t_begin; t < t_end; ++t) {
       // the place of turn t + 1 was read in turn t - 1, which everyone has left
-      if (t + 1 < n_turns) stash(split_lds + ((t + 1) & 1) * SPLIT_TURN);
-      if (t + 2 < n_turns) fetch(t + 2);
+      if (t + 1 < t_end) stash(split_lds + ((t + 1 - t_begin) & 1) * SPLIT_TURN);
+      if (t + 2 < t_end) fetch(t + 2);
       __syncthreads();                                       // the end of turn t
     }
     __syncthreads();                                         // (before the second set's results are read)
@@ -616,12 +628,24 @@ attention_prefill_split_kernel(AttnArgs a) {
   const float c = a.scale * LOG2_E;
   const int whole_until = start + q0 + 1;       // blocks ending here or before are seen whole
 
+  if (empty_run) {       // a run beyond the tile's last turn: its records say that it saw no key
+    if (set == 0 && g == 0) {
+#pragma unroll
+      for (int nq = 0; nq < PREFILL_NQ; ++nq)
+        if (qpos[nq] >= 0) {
+          float* record = a.partial + (((int64_t)tok[nq] * a.q_heads + head) * runs + run) * (HD + 2);
+          record[HD] = -INFINITY;
+          record[HD + 1] = 0.f;
+        }
+    }
+    return;
+  }
   __syncthreads();                              // the first turn is in place
-  for (int t = 0; t < n_turns; ++t) {
+  for (int t = t_begin; t < t_end; ++t) {
     const int block_index = 2 * t + set;
     const int kb = block_index * BT_KV_BLOCK;
     if (block_index < n_blocks && kb < hi) {
-      const unsigned char* stage = split_lds + (t & 1) * SPLIT_TURN + set * SHARED_STAGE;
+      const unsigned char* stage = split_lds + ((t - t_begin) & 1) * SPLIT_TURN + set * SHARED_STAGE;
       BlockOperands blk;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
@@ -670,6 +694,24 @@ attention_prefill_split_kernel(AttnArgs a) {
     const float total = rows[nq][0] * mine + l_other * theirs;   // (whole sums: see attend_block)
     float inv = total > 0.f ? 1.0f / total : 0.f;
     if (qpos[nq] < 0) continue;
+    if (runs > 1) {      // this run's share of the query's row, relative to its own maximum
+      typedef __attribute__((__vector_size__(2 * sizeof(float)))) float float2v;
+      float* record = a.partial + (((int64_t)tok[nq] * a.q_heads + head) * runs + run) * (HD + 2);
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt) {
+        float joined[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          joined[r] = o[nq][dt][r] * mine + hand[((k0 + 2 + 4 * dt + r) * PREFILL_WAVES + wave) * 64 + lane] * theirs;
+        *reinterpret_cast<float2v*>(record + dt * 16 + 4 * g) = float2v{joined[0], joined[1]};
+        *reinterpret_cast<float2v*>(record + dt * 16 + 4 * g + 2) = float2v{joined[2], joined[3]};
+      }
+      if (g == 0) {
+        record[HD] = top;
+        record[HD + 1] = total;
+      }
+      continue;
+    }
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt) {
       float joined[4];
@@ -808,7 +850,9 @@ attention_decode_kernel(AttnArgs a) {
   }
 }
 
-// Joins the runs of attention_decode_kernel: a work-group of one wave per (sequence, query head).
+// Joins the runs of attention_decode_kernel (a row is a sequence's one token) or of
+// attention_prefill_split_kernel (a row is a token of the step): a work-group of one wave per
+// (row, query head).  A run that saw no key has the maximum -inf and whatever else in its record.
 __global__ void __launch_bounds__(64)
 attention_join_kernel(AttnArgs a) {
   const int seq = blockIdx.x / a.q_heads, head = blockIdx.x % a.q_heads;
@@ -820,7 +864,9 @@ attention_join_kernel(AttnArgs a) {
     float num = 0.f, den = 0.f;
     if (top != -INFINITY) {
       for (int s = 0; s < a.splits; ++s) {
-        float f = exp2f(runs[s * (HD + 2) + HD] - top);
+        const float m_run = runs[s * (HD + 2) + HD];
+        if (m_run == -INFINITY) continue;
+        float f = exp2f(m_run - top);
         num += runs[s * (HD + 2) + channel] * f;
         den += runs[s * (HD + 2) + HD + 1] * f;
       }
@@ -850,6 +896,10 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
   int rc = check_args(*args, "attention_prefill_bf16");
   if (rc) return rc;
   if (args->max_count <= 0) BT_REFUSE("attention_prefill_bf16: max_count %d must be positive", args->max_count);
+  const int runs = args->splits > 1 ? args->splits : 1;
+  if (runs > 1 && (HD != 64 || args->window != 0 || !args->partial || runs > 64))
+    BT_REFUSE("attention_prefill_bf16: runs of keys (%d) are for heads of 64 without a window, at most 64, and need a place "
+              "for their partial results", runs);
   const int q_tiles = (args->max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES;
   const int group = args->q_heads / args->kv.kv_heads;
   const int64_t units = (int64_t)args->n_seqs * args->kv.kv_heads;
@@ -874,10 +924,16 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
       if (err != hipSuccess) BT_REFUSE("attention_prefill_bf16: cannot get %d bytes of LDS: %s", (int)SPLIT_LDS_BYTES, hipGetErrorString(err));
       raised = true;
     }
-    const int64_t split_groups = 8 * units_per_xcd * group * q_tiles;
+    const int64_t split_groups = 8 * ((units * runs + 7) / 8) * group * q_tiles;
     if (split_groups > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: %lld work-groups are too many", (long long)split_groups);
     hipLaunchKernelGGL(attention_prefill_split_kernel, dim3((unsigned)split_groups), dim3(SPLIT_THREADS), SPLIT_LDS_BYTES,
                        (hipStream_t)stream, *args);
+    if (runs > 1) {
+      rc = bt_check_launch("attention_prefill_bf16");
+      if (rc) return rc;
+      if ((int64_t)args->n_tokens * args->q_heads > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: too many rows to join");
+      hipLaunchKernelGGL(attention_join_kernel, dim3((unsigned)args->n_tokens * args->q_heads), dim3(64), 0, (hipStream_t)stream, *args);
+    }
     return bt_check_launch("attention_prefill_bf16");
   }
 #endif

@@ -750,17 +750,20 @@ def _library_has_algorithm(lda, m, n, k, epilogue):
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
-                   scale, window=0, partial=None):
-    """``partial``: float32 [n_seqs * q_heads * runs, head_dim + 2] for a decode step whose keys are
-    cut into runs that separate work-groups take (long contexts in small batches).  ``out`` may be a
-    :class:`Chunked` for the bfloat16 decode kernels."""
+                   scale, window=0, partial=None, runs=None):
+    """``partial``: float32 [rows * q_heads * runs, head_dim + 2] for a step whose keys are cut into
+    runs that separate work-groups take.  Decode steps (long contexts in small batches): rows are
+    the sequences, and ``runs`` follows from the shape.  Prompt steps (few query tiles behind a long
+    context): rows are the step's tokens, the buffer may be longer than this step needs, and
+    ``runs`` is given.  ``out`` may be a :class:`Chunked` for the bfloat16 decode kernels."""
     splits = 1
     if partial is not None:
-        splits = partial.shape[0] // (n_seqs * q_heads)
+        rows = n_seqs if runs is None else q.shape[0]
+        splits = partial.shape[0] // (rows * q_heads) if runs is None else runs
         if partial.dtype != torch.float32 or not partial.is_contiguous() or partial.shape[1] != kv_view.head_dim + 2 \
-                or splits * n_seqs * q_heads != partial.shape[0]:
+                or (splits * rows * q_heads != partial.shape[0] if runs is None else splits * rows * q_heads > partial.shape[0]):
             raise KernelError(f"attention: partial results of shape {tuple(partial.shape)} do not fit "
-                              f"{n_seqs} sequences of {q_heads} heads of {kv_view.head_dim}")
+                              f"{rows} rows of {q_heads} heads of {kv_view.head_dim} in {splits} runs")
     return AttnArgs(splits=splits, partial=partial.data_ptr() if partial is not None and splits > 1 else None,
                     q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0), out_rows=_out_rows(out),
                     tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), seq_off=seq_off.data_ptr(),

@@ -30,6 +30,9 @@ from .registry import register
 # compute units, at least RUN_BYTES of keys and values per run, and no cut below SPLIT_BYTES.
 SPLIT_BYTES = 384 << 10
 RUN_BYTES = 128 << 10
+# A prompt step with few tiles of queries (a chunk of a prompt) cuts the keys of every tile into runs
+# of at least this many blocks of 64 keys for every 256 tokens of the step (prompt_runs).
+PROMPT_RUN_BLOCKS = 8
 
 
 @register("mixer", "attention")
@@ -98,6 +101,18 @@ class CausalSelfAttention(Mixer):
         pairs = step.n_seqs * self.kv_heads
         return max(1, min(compute_units(device) // pairs, pair_bytes // RUN_BYTES, 64))
 
+    def prompt_runs(self, step, device):
+        """Into how many runs a prompt step's query tiles cut their keys: a chunk of a prompt behind
+        a long context has few tiles of 128 queries (a work-group each) and many keys for each, so
+        the keys are shared out until the work-groups fill the chip, a run keeping at least
+        ``PROMPT_RUN_BLOCKS`` blocks of keys.  Planned from what the steps of one class of token
+        counts share (most tokens, sequences, most blocks of a sequence), like ``decode_runs``."""
+        if step.decode or not step.dtype_is_bf16 or self.head_dim != 64 or self.window or self.plain_only:
+            return 1
+        tiles = -(-step.token_capacity // 128) + step.n_seqs - 1          # at most so many hold queries
+        blocks = PROMPT_RUN_BLOCKS * -(-step.token_capacity // 256)       # (joining costs by the token)
+        return max(1, min(compute_units(device) // (tiles * self.heads), step.max_blocks // blocks, 8))
+
     def forward(self, h, step, memory, stream):
         tokens = h.shape[0]
         kv = memory.kv()
@@ -124,10 +139,13 @@ class CausalSelfAttention(Mixer):
             mixed = K.Chunked.take(step, "attention.mixed", tokens, self.n_q, step.dtype)    # the layout the next product reads fastest
         else:
             mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
-        partial, runs = None, self.decode_runs(step, h.device)
+        partial, runs, prompt_runs = None, self.decode_runs(step, h.device), self.prompt_runs(step, h.device)
         if runs > 1:
             partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")
+        elif prompt_runs > 1:
+            partial = step.buffer("attention.partial", tokens * self.heads * prompt_runs, self.head_dim + 2, "float32")
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
-                                self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial)
+                                self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial,
+                                runs=prompt_runs if prompt_runs > 1 else None)
         K.attention(args, step.dtype, step.decode, impl="plain" if self.plain_only else "auto")
         stream.add_product(step, mixed, self.out_weight, self.out_bias, packed=self.out_packed)

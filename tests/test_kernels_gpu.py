@@ -660,6 +660,66 @@ def test_attention_decode_in_runs(dtype, hd, window):
                          q_heads, len(totals), 1, 1.0, window, torch.zeros(7, hd + 2, device=DEV))
 
 
+@pytest.mark.parametrize("q_heads,kv_heads", [(2, 2), (4, 2)])
+def test_prompt_attention_in_runs_of_keys(q_heads, kv_heads):
+    """A chunk of a prompt behind a long context has few tiles of queries and many keys for each: the
+    keys of every tile are cut into runs that separate work-groups take and a second kernel joins.
+    Every number of runs gives what the undivided kernel gives (a chunk that starts off the block
+    grid, a sequence with nothing behind its chunk, one shorter than a tile, runs that are empty for
+    the early tiles), queries that look at ONE key find it in whichever run it falls, and the
+    records are written into a buffer full of NaN, longer than the step needs."""
+    dt, hd = torch.bfloat16, 64
+    totals, counts = [3000, 300, 1183, 70], [256, 300, 200, 3]
+    case = PagedCase(totals, counts, kv_heads, hd, dt, DEV, seed=31, poison=True)
+    gen = torch.Generator().manual_seed(32)
+    q = torch.randn(case.n_tokens, q_heads * hd, generator=gen) * 0.3
+    # queries of sequence 0 (positions 2744 ...): row 5 of head 0 looks at key 9 alone, row 130 at
+    # key 1500, row 255 of the last head at its own position, row 200 at key 2688 (its tile's last block but one)
+    group = q_heads // kv_heads
+    targets = [(0, 5, 0, 9), (0, 130, 0, 1500), (0, 255, q_heads - 1, 2999), (0, 200, 0, 2688)]
+    offsets = [0]
+    for c in counts:
+        offsets.append(offsets[-1] + c)
+    for s, row, head, key in targets:
+        kv_head = head // group
+        case.k_rows[s][:, kv_head * hd:(kv_head + 1) * hd] *= 0.05
+    for index, (s, row, head, key) in enumerate(targets):      # (a channel of its own for each, so that no query sees two)
+        kv_head = head // group
+        case.k_rows[s][key, kv_head * hd + 3 + 5 * index] = 8.0
+        q[offsets[s] + row, head * hd:(head + 1) * hd] = 0.0
+        q[offsets[s] + row, head * hd + 3 + 5 * index] = 8.0
+    seq = torch.cat([torch.full((t,), i, dtype=torch.int32) for i, t in enumerate(totals)]).to(DEV)
+    pos = torch.cat([torch.arange(t, dtype=torch.int32) for t in totals]).to(DEV)
+    K.kv_copy(torch.cat(case.k_rows).to(DEV), torch.cat(case.v_rows).to(DEV), seq, pos, case.view(), True)
+    q = q.to(dt).to(DEV)
+    want = case.reference(q, q_heads, 1.0, 0)
+    for s, row, head, key in targets:
+        kv_head = head // group
+        value = case.v_rows[s][key, kv_head * hd:(kv_head + 1) * hd].double()
+        assert (want[offsets[s] + row, head * hd:(head + 1) * hd] - value).abs().max() < 2e-3, (row, key)
+    results = {}
+    for runs in (1, 2, 3, 8, 64):
+        out = torch.full((case.n_tokens, q_heads * hd), float("nan"), dtype=dt, device=DEV)
+        partial = torch.full(((case.n_tokens + 9) * q_heads * runs, hd + 2), float("nan"), device=DEV) if runs > 1 else None
+        args = K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                                q_heads, len(totals), max(counts), 1.0, 0, partial, runs=runs if runs > 1 else None)
+        K.attention(args, dt, decode=False, impl="mfma")
+        assert rel_err(out, want) < 1.2e-2, runs
+        for s, row, head, key in targets:
+            got = out[offsets[s] + row, head * hd:(head + 1) * hd].double().cpu()
+            assert (got - want[offsets[s] + row, head * hd:(head + 1) * hd].cpu()).abs().max() < 3e-2, (runs, row, key)
+        results[runs] = out
+    # runs are refused where the kernel that takes them does not run: a window, another head size
+    partial = torch.zeros(case.n_tokens * q_heads * 2, hd + 2, device=DEV)
+    args = K.attention_args(q, results[1].clone(), case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                            q_heads, len(totals), max(counts), 1.0, 100, partial, runs=2)
+    with pytest.raises(K.KernelError, match="runs of keys"):
+        K.attention(args, dt, decode=False, impl="mfma")
+    with pytest.raises(K.KernelError, match="do not fit"):
+        K.attention_args(q, out, case.view(), case.tok_seq, case.tok_pos, case.seq_off, case.seq_start,
+                         q_heads, len(totals), max(counts), 1.0, 0, torch.zeros(7, hd + 2, device=DEV), runs=2)
+
+
 @pytest.mark.parametrize("pattern", ["ramp", "jumps", "falling"])
 def test_attention_with_scores_that_rise_and_jump(pattern):
     """The running maximum is allowed to lag a little before sums are rescaled: scores that creep

@@ -178,6 +178,51 @@ def test_unequal_batches_one_after_another(dtype):
 
 # --- GPT-2 small's sizes with all twelve layers, in float32 and in bfloat16: depth ----------------
 
+LONG = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "n_embd": 256, "n_head": 4,
+        "n_inner": 512, "vocab_size": 1000, "n_positions": 4096, "activation_function": "gelu_new",
+        "layer_norm_epsilon": 1e-5, "scale_attn_by_inverse_layer_idx": False}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_chunks_of_a_prompt_behind_a_long_context(dtype):
+    """A request of 3,300 tokens fed in chunks of 256 (heads of 64, room for 4,096 positions, attention
+    sharpened): from the third chunk on the bfloat16 attention kernel cuts the keys of its two query
+    tiles into runs that separate work-groups take and a second kernel joins.  The logits at the
+    first, a middle and the last place of every chunk against the plain implementation, and a
+    second request beside it whose chunks are shorter than a tile."""
+    from types import SimpleNamespace
+    with tempfile.TemporaryDirectory(prefix="bt_long_") as folder:
+        weights = bt.write_random_model(folder, LONG, 12)
+        d = LONG["n_embd"]
+        for layer in range(LONG["n_layer"]):
+            weights[f"h.{layer}.attn.c_attn.weight"][:, :2 * d] *= 4.0
+            weights[f"h.{layer}.attn.c_attn.bias"][:2 * d] *= 4.0
+        stored = {k: (v.to(torch.bfloat16) if v.dim() == 2 else v) for k, v in weights.items()}
+        bt.write_safetensors(os.path.join(folder, "model.safetensors"), stored)
+        weights = {k: v.float() for k, v in stored.items()}
+        model = bt.load_model(folder, dtype=dtype, device="cuda:0")
+    mixer = model.blocks[0].mixers()[0]
+    late = SimpleNamespace(decode=False, dtype_is_bf16=dtype == "bfloat16", token_capacity=256, n_seqs=1, max_blocks=52)
+    assert mixer.prompt_runs(late, "cuda:0") == (6 if dtype == "bfloat16" else 1)      # (what the test is about)
+    engine = bt.Engine(model, max_tokens=4096 + 512)
+    gen = torch.Generator().manual_seed(13)
+    requests = [torch.randint(0, LONG["vocab_size"], (n,), generator=gen).tolist() for n in (3300, 900)]
+    chunks, fed, slots = [256, 70], [0, 0], [engine.open(), engine.open()]
+    got, rows = [[], []], [[], []]
+    while any(f < len(r) for f, r in zip(fed, requests)):
+        live = [i for i in range(2) if fed[i] < len(requests[i])]
+        entries = [(slots[i], requests[i][fed[i]:fed[i] + chunks[i]]) for i in live]
+        wants = [[0, len(e[1]) // 2, len(e[1]) - 1] for e in entries]
+        logits = engine.step(entries, want=wants).clone()
+        for n, i in enumerate(live):
+            got[i].append(logits[3 * n:3 * n + 3])
+            rows[i] += [fed[i] + w for w in wants[n]]
+            fed[i] += len(entries[n][1])
+    for i, r in enumerate(requests):
+        want = plain.forward(r, weights, LONG, rows=rows[i])
+        check(torch.cat(got[i]), want, dtype, f"request {i} of {len(r)} tokens in chunks of {chunks[i]}")
+
+
 SMALL = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 12, "n_embd": 768, "n_head": 12,
          "n_inner": 3072, "vocab_size": 50257, "n_positions": 1024, "activation_function": "gelu_new",
          "layer_norm_epsilon": 1e-5, "scale_attn_by_inverse_layer_idx": False}

@@ -284,9 +284,9 @@ class Engine:
             # (measurements under way were of lists that are gone; decisions taken stay)
             self._launch_bound = {k: v for k, v in self._launch_bound.items() if isinstance(v, bool)}
         layout = plan.layout
-        exact = (layout.key(), plan.max_count, readout, plan.context_limit if plan.decode else 0)
+        exact = (layout.key(), plan.max_count, readout, plan.context_limit)
         # a step of more than 64 tokens that is not one of single tokens shares its list with its class
-        shared = (layout.class_key(), readout) if layout.tokens > BLOCK and plan.max_count > 1 else None
+        shared = (layout.class_key(), readout, plan.context_limit) if layout.tokens > BLOCK and plan.max_count > 1 else None
         key = shared if shared is not None and shared in self._programs else exact
         held = self._programs.pop(key, None)
         if held is not None:
@@ -335,8 +335,8 @@ class Engine:
         return logits
 
     def _run_from_graph(self, plan, readout):
-        # (parts plan decode steps by the class of context; steps with prompt tokens look the same in every class)
-        key = (plan.layout.key(), plan.max_count, readout, plan.context_limit if plan.decode else 0)
+        # (parts plan by the class of context: how many runs the keys of a decode step or of a chunk are cut into)
+        key = (plan.layout.key(), plan.max_count, readout, plan.context_limit)
         held = self._graphs.pop(key, None)
         if held is not None and held["generation"] != self.pool.generation:
             held = None                                   # a workspace moved: the graph is stale
@@ -380,7 +380,7 @@ class Engine:
             if len(self._launch_bound) > 4096:
                 self._launch_bound.clear()
             probe = self._launch_bound[key] = []
-        shared = (plan.layout.class_key(), readout)
+        shared = (plan.layout.class_key(), readout, plan.context_limit)
         if key not in self._programs and shared not in self._programs and self._seen.get(key, 0) < 8:
             # the shape has no list (its first step made a workspace grow, or the lists were dropped
             # since): this step would be launched from Python and say nothing about the list; it

@@ -33,6 +33,7 @@ RUN_BYTES = 128 << 10
 # A prompt step with few tiles of queries (a chunk of a prompt) cuts the keys of every tile into runs
 # of at least this many blocks of 64 keys for every 256 tokens of the step (prompt_runs).
 PROMPT_RUN_BLOCKS = 8
+PROMPT_RUN_MIN_CONTEXT = 1024      # no runs in steps whose class of context is this or less: they gain from some 2,000 keys on
 
 
 @register("mixer", "attention")
@@ -105,13 +106,19 @@ class CausalSelfAttention(Mixer):
         """Into how many runs a prompt step's query tiles cut their keys: a chunk of a prompt behind
         a long context has few tiles of 128 queries (a work-group each) and many keys for each, so
         the keys are shared out until the work-groups fill the chip, a run keeping at least
-        ``PROMPT_RUN_BLOCKS`` blocks of keys.  Planned from what the steps of one class of token
-        counts share (most tokens, sequences, most blocks of a sequence), like ``decode_runs``."""
+        ``PROMPT_RUN_BLOCKS`` blocks of keys.  Planned from what the steps that share a launch list
+        have in common (most tokens, sequences, the class of context), like ``decode_runs``.
+        Measured at 25 heads of 64, a chunk of 256 tokens, us a call with 1 / 2 / 4 / 5 runs: behind
+        1,024 tokens 16.6 / 16.9 / 17.3 / 18.0, 2,048: 25.9 / 21.9 / 20.4 / 20.8, 4,096: 45.7 / 31.9 /
+        25.5 / 25.3, 8,192: 84.5 / 51.9 / 35.6 / 33.7; two sequences (100 work-groups) 4,096: 48.1 /
+        36.9, 8,192: 88.4 / 57.7."""
         if step.decode or not step.dtype_is_bf16 or self.head_dim != 64 or self.window or self.plain_only:
+            return 1
+        if step.context_limit <= PROMPT_RUN_MIN_CONTEXT:
             return 1
         tiles = -(-step.token_capacity // 128) + step.n_seqs - 1          # at most so many hold queries
         blocks = PROMPT_RUN_BLOCKS * -(-step.token_capacity // 256)       # (joining costs by the token)
-        return max(1, min(compute_units(device) // (tiles * self.heads), step.max_blocks // blocks, 8))
+        return max(1, min(compute_units(device) // (tiles * self.heads), step.context_limit // (64 * blocks), 8))
 
     def forward(self, h, step, memory, stream):
         tokens = h.shape[0]

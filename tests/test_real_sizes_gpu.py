@@ -186,7 +186,7 @@ LONG = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_chunks_of_a_prompt_behind_a_long_context(dtype):
     """A request of 3,300 tokens fed in chunks of 256 (heads of 64, room for 4,096 positions, attention
-    sharpened): from the third chunk on the bfloat16 attention kernel cuts the keys of its two query
+    sharpened): from 1,024 tokens of context on the bfloat16 attention kernel cuts the keys of its two query
     tiles into runs that separate work-groups take and a second kernel joins.  The logits at the
     first, a middle and the last place of every chunk against the plain implementation, and a
     second request beside it whose chunks are shorter than a tile."""
@@ -202,8 +202,10 @@ def test_chunks_of_a_prompt_behind_a_long_context(dtype):
         weights = {k: v.float() for k, v in stored.items()}
         model = bt.load_model(folder, dtype=dtype, device="cuda:0")
     mixer = model.blocks[0].mixers()[0]
-    late = SimpleNamespace(decode=False, dtype_is_bf16=dtype == "bfloat16", token_capacity=256, n_seqs=1, max_blocks=52)
-    assert mixer.prompt_runs(late, "cuda:0") == (6 if dtype == "bfloat16" else 1)      # (what the test is about)
+    late = SimpleNamespace(decode=False, dtype_is_bf16=dtype == "bfloat16", token_capacity=256, n_seqs=1, context_limit=4096)
+    assert mixer.prompt_runs(late, "cuda:0") == (8 if dtype == "bfloat16" else 1)      # (what the test is about)
+    early = SimpleNamespace(decode=False, dtype_is_bf16=dtype == "bfloat16", token_capacity=256, n_seqs=1, context_limit=1024)
+    assert mixer.prompt_runs(early, "cuda:0") == 1
     engine = bt.Engine(model, max_tokens=4096 + 512)
     gen = torch.Generator().manual_seed(13)
     requests = [torch.randint(0, LONG["vocab_size"], (n,), generator=gen).tolist() for n in (3300, 900)]

@@ -714,7 +714,11 @@ def deep_split_count(rows, columns, k, units=256):
     units (us for 1600 x 1600 and 1600 x 6400, slices 2 / 3 / 4): 128 rows 7.1 / 6.3 / 5.9 and 18.9 /
     14.5 / 12.1; 192 rows 7.3 / 6.5 / 7.2 and 18.8 / 14.7 / 18.8; 256 rows 7.4 / 7.9 / 7.5 and 19.2 /
     22.4 / 18.8; 384 rows 9.3 / 8.4 / 10.9 and 29.3 / 23.1 / 26.5; 512 rows 9.5 / 12.1 / 12.1 and 30.7 /
-    32.2 / 31.0 (the vendor's library: 11.1 to 12.2 and 18.3 to 32.4)."""
+    32.2 / 31.0 (the vendor's library: 11.1 to 12.2 and 18.3 to 32.4).  Measured and not taken: tiles
+    of 128 x 128 in four slices for 1600 x 6400 at 512 rows (25.2 us alone against 30.3, but 29.5 in
+    the step, where the norm behind it also reads four slices instead of two), and slices beyond 512
+    rows (640 rows: 10.1 and 30.7 against the library's 12.2 and 32.7, which the norm's second
+    reading of two slices takes back)."""
     if not deep_form_rows(rows, k, k, columns, sliced=True):
         return 1
     tiles = ((rows + 63) // 64) * ((columns + 63) // 64)

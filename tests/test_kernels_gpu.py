@@ -261,7 +261,8 @@ def test_skinny_gemm_normalises_its_rows_itself(m, n, k, kind, with_shift, colum
 
 
 @pytest.mark.parametrize("impl,m,n,k,splits", [("skinny", 5, 96, 1600, 4), ("skinny", 64, 50, 6400, 8),
-                                               ("skinny", 20, 1600, 320, 2), ("tile", 150, 200, 1600, 3)])
+                                               ("skinny", 20, 1600, 320, 2), ("tile", 150, 200, 1600, 3),
+                                               ("tile", 600, 1600, 6400, 3), ("tile", 512, 1600, 6400, 4)])
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 def test_gemm_split_k_partials(impl, m, n, k, splits, dtype):
     a, w, bias, want = operands(m, n, k, DTYPES[dtype], seed=splits)
@@ -768,7 +769,8 @@ def test_add_norm(dtype, width, rows):
     dt = DTYPES[dtype]
     gen = torch.Generator().manual_seed(width)
     x = (torch.randn(rows, width, generator=gen) * 2 + 0.5).to(DEV)
-    delta = torch.randn(3, rows, width, generator=gen).to(DEV)
+    more = torch.randn(5, rows, width, generator=gen).to(DEV)
+    delta = more[:3].contiguous()
     bias = torch.randn(width, generator=gen).to(DEV)
     gamma = (1 + 0.1 * torch.randn(width, generator=gen)).to(DEV)
     beta = torch.randn(width, generator=gen).to(DEV)
@@ -780,6 +782,13 @@ def test_add_norm(dtype, width, rows):
     K.add_norm(xs, out, gamma, beta, 1e-3, "layer_norm", delta=delta, bias=bias)
     assert rel_err(out, want) < tol
     assert rel_err(xs, total) < 1e-6
+    # other numbers of pending sums (the wave-per-row kernel has a form for each up to four, and a loop)
+    for n in (1, 2, 4, 5):
+        xs = x.clone()
+        K.add_norm(xs, out, gamma, beta, 1e-3, "layer_norm", delta=more[:n].contiguous(), bias=bias)
+        summed = x.double() + more[:n].double().sum(0) + bias.double()
+        assert rel_err(xs, summed) < 1e-6, n
+        assert rel_err(out, torch.nn.functional.layer_norm(summed, (width,), gamma.double(), beta.double(), 1e-3)) < tol, n
     # selected rows: nothing is written back
     pick = torch.tensor([rows - 1, 0], dtype=torch.int32, device=DEV)
     xs = x.clone()

@@ -21,8 +21,8 @@ One JSON line is printed:
   spread      milliseconds per step of the fastest, median and slowest repetition
   prefill     one step of 2 x 1,024 prompt tokens: tokens/s, ms, fraction of the MFMA peak;
               `own` is the same step with every product on this package's kernels (the default
-              hands products of more than 64 rows to hipBLASLt, as the reference hands its
-              products to its backend's library)
+              hands products of more than 256 rows, 512 for those that add to the residual
+              stream, to hipBLASLt, as the reference hands its products to its backend's library)
   roofline    bytes a decode step has to read (every weight once + the live cache) / its time,
               against 8 TB/s
   points      decoded tokens per second at batch 1 and 64, at batch 8 from prompts of 896 tokens
@@ -310,7 +310,7 @@ def run_xl(args):
                "ms": round(1000.0 * prefill_seconds, 3),
                "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[args.dtype], 4),
                "min_ms": round(1000.0 * prefill_times[0], 3), "max_ms": round(1000.0 * prefill_times[-1], 3),
-               "products": "hipBLASLt beyond 64 rows" if args.dtype == "bf16" and K.library_products() else "own kernels"}
+               "products": "hipBLASLt beyond 256 rows" if args.dtype == "bf16" and K.library_products() else "own kernels"}
     kernels = {}
     if not args.no_kernels:
         kernels["decode"] = decode_kernels(engine, args.batch, vocab, config, args.dtype, int(mean_context))

@@ -430,8 +430,9 @@ def library_products():
 
     The reference leaves its matrix products to its backend's library (src/attention.rs:481-513
     and the feed-forward call ``linear``); here the vendor's library takes the products of steps
-    with more than 64 rows, where it is about 1.6 times as fast as the tile kernel of this
-    package at GPT-2 XL sizes, and the hand-written kernels keep everything else.  The library is
+    with more than 256 rows (512 for those that add to the residual stream: ``deep_form_rows``),
+    where it is about 1.6 times as fast as the tile kernel of this package at GPT-2 XL sizes, and
+    the hand-written kernels keep everything else.  The library is
     opened from the copy that came with torch's HIP runtime and checked once against the tile
     kernel; if it cannot be opened, or disagrees, the tile kernel does those products too, and
     a line on stderr says so.

@@ -492,9 +492,13 @@ gemm_tile_dma_kernel(const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __
 // together pull at 6 to 12 TB/s through the L2s, more the more of them share a compute unit; a
 // kernel that only reads as much without a loop does 27 TB/s from the L2 and 6.6 from memory.
 // For prompts of thousands of rows a tile of 256 x 256 on eight waves (twice the multiplications
-// per byte pulled) was measured too: its two stages of 64 KiB are all that the LDS holds, so one
-// tile is in flight at a time, and 2048 x 4800 x 1600 took 86 us where the lean form takes 70 and
-// the vendor's library 39.
+// per byte pulled) was measured too, in two forms.  With K in steps of 64 its two stages of 64 KiB
+// are all that the LDS holds, so one tile is in flight at a time and its latency is not hidden:
+// 2048 x 4800 x 1600 took 86 us where the lean form takes 70 and the vendor's library 39.  With K in
+// steps of 32 and four stages of 32 KiB (rows two to a 128-byte line, swizzled free of bank
+// conflicts) three tiles are in flight, but a wave's load then asks for sixteen half cache lines
+// where it asked for eight whole ones, and a compute unit pulls half the bytes: 88 us.  What a
+// compute unit pulls is a number of cache lines a microsecond (about 300), not of bytes.
 template <int NEWER, int LOADS>
 __device__ __forceinline__ void wait_for_all_but(int newer) {
   // waits until at most `newer` tiles' loads (LOADS instructions each) of this wave are in flight

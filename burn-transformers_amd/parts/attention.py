@@ -28,6 +28,9 @@ from .registry import register
 # 8,192 keys 47.7 / 29.6 / 23.0 / 19.3 / 23.6; eight sequences (200 pairs of sequence and head
 # already) lose with any cut, 73 / 80 / 85 us at 8,192 keys.  So: no more work-groups than
 # compute units, at least RUN_BYTES of keys and values per run, and no cut below SPLIT_BYTES.
+# (With the joining kernel that asks for eight runs' records at once, one sequence measures 7.1 us
+# in eight runs at 1,024 keys where one run takes 8.8; in the step that gained 0.2 % at batch 1,
+# the second kernel's place in the chain costing what its work-groups save: not taken.)
 SPLIT_BYTES = 384 << 10
 RUN_BYTES = 128 << 10
 # A prompt step with few tiles of queries (a chunk of a prompt) cuts the keys of every tile into runs

@@ -1,7 +1,9 @@
-"""Two more toy parts, defined and registered here without touching the library's files: a
-feed-forward that routes (two experts mixed by a softmax gate computed in float32) and a
-position encoding of another kind (sinusoids added to the token embedding).  Both work on
-device tensors only, so the engine replays their decode steps from a HIP graph like GPT-2's."""
+"""More toy parts, defined and registered here without touching the library's files: a
+feed-forward that routes (two experts mixed by a softmax gate computed in float32), a position
+encoding of another kind (sinusoids added to the token embedding), and, in a second model, a
+norm of another kind (by the mean absolute value) with a readout that has a table of its own, a
+bias and a soft cap.  All work on device tensors only, so the engine replays their decode steps
+from a HIP graph like GPT-2's."""
 
 from dataclasses import dataclass
 
@@ -14,7 +16,7 @@ import burn_transformers_amd as bt  # noqa: E402
 import plain_gpt2 as plain  # noqa: E402
 from burn_transformers_amd.engine.plan import LayerPlan, ModelPlan, PartSpec, ScheduleEntry  # noqa: E402
 from burn_transformers_amd.kernels import library as K  # noqa: E402
-from burn_transformers_amd.parts import Delta, Embedding, FeedForward, ResidualStream, register, unregister  # noqa: E402
+from burn_transformers_amd.parts import Delta, Embedding, FeedForward, Norm, Readout, ResidualStream, register, unregister  # noqa: E402
 
 
 class GatedExperts(FeedForward):
@@ -169,3 +171,140 @@ def test_routed_feed_forward_and_sinusoid_positions(dtype, tmp_path):
         unregister("feed_forward", "toy_gated_experts")
         unregister("embedding", "toy_sinusoid")
         bt.unregister_family("toy_routed")
+
+
+class MeanAbsNorm(Norm):
+    """y = x / (mean |x| + eps) * scale: statistics in float32 on what the stream holds once the
+    pending sums are added."""
+
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        self.eps, self.scale = params["eps"], tensors["weight"]
+
+    def apply(self, stream, step, rows=None):
+        stream.flush()                                   # (adds what the part before left pending)
+        x = stream.x if rows is None else stream.x[rows.long()]
+        y = x / (x.abs().mean(dim=-1, keepdim=True) + self.eps) * self.scale
+        return y.to(step.dtype)
+
+
+class CappedReadout(Readout):
+    """logits = cap * tanh((h . table^T + bias) / cap): a table of its own, a bias and a soft cap."""
+
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        self.cap, self.table, self.bias = params["cap"], tensors["weight"], tensors["bias"]
+
+    def logits(self, h, step):
+        out = step.buffer("toy.logits", h.shape[0], self.table.shape[0], "float32")
+        K.gemm(h, self.table, K.epilogue_f32(out, self.bias))
+        return self.cap * torch.tanh(out / self.cap)
+
+
+@dataclass(frozen=True)
+class CappedConfig:
+    width: int = 64
+    inner: int = 72
+    vocab_size: int = 53
+    max_positions: int = 96
+    heads: int = 2
+    cap: float = 3.0
+    eps: float = 1e-3
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(**{k: data[k] for k in cls.__dataclass_fields__ if k in data})
+
+    def to_dict(self):
+        return dict(architectures=["ToyCappedLM"], **{k: getattr(self, k) for k in self.__dataclass_fields__})
+
+
+def capped_plan(c):
+    hd = c.width // c.heads
+    norm = lambda p: PartSpec("toy_mean_abs_norm", {"width": c.width, "eps": c.eps}, {"weight": p})
+    attention = PartSpec("attention", {"width": c.width, "heads": c.heads, "kv_heads": c.heads, "head_dim": hd,
+                                       "scale": hd ** -0.5, "window": 0}, {"qkv_weight": "qkv", "out_weight": "out"})
+    ff = PartSpec("dense", {"width": c.width, "inner": c.inner, "activation": "gelu_tanh"},
+                  {"up_weight": "up", "up_bias": "up.b", "down_weight": "down", "down_bias": "down.b"})
+    layer = LayerPlan("pre_norm", {"mixer_norm": norm("n1"), "mixer": attention, "ff_norm": norm("n2"), "ff": ff})
+    return ModelPlan(c.width, c.vocab_size, c.max_positions,
+                     PartSpec("learned_positions", {"width": c.width, "vocab_size": c.vocab_size,
+                                                    "max_positions": c.max_positions}, {"tokens": "tok", "positions": "pos"}),
+                     [layer, layer], [ScheduleEntry(0, 0), ScheduleEntry(1, 1)], norm("final"),
+                     PartSpec("toy_capped_readout", {"cap": c.cap}, {"weight": "head", "bias": "head.b"}))
+
+
+def capped_contract(c):
+    d = c.width
+    specs = [("tok", (c.vocab_size, d), "table"), ("pos", (c.max_positions, d), "table"), ("head", (c.vocab_size, d), "out_in"),
+             ("head.b", (c.vocab_size,), "vector"), ("qkv", (3 * d, d), "out_in"), ("out", (d, d), "out_in"),
+             ("up", (c.inner, d), "out_in"), ("up.b", (c.inner,), "vector"), ("down", (d, c.inner), "out_in"),
+             ("down.b", (d,), "vector"), ("n1", (d,), "vector"), ("n2", (d,), "vector"), ("final", (d,), "vector")]
+    return bt.Contract([bt.TensorSpec(*s) for s in specs])
+
+
+def capped_init(c, generator):
+    out = {}
+    for spec in capped_contract(c).tensors:
+        t = torch.randn(spec.shape, generator=generator)
+        if spec.layout == "vector":
+            out[spec.name] = 1 + 0.2 * t if spec.name in ("n1", "n2", "final") else 0.3 * t
+        else:
+            out[spec.name] = t * (0.5 if spec.layout == "table" else spec.shape[-1] ** -0.5)
+    out["head"] *= 4.0          # logits beyond the cap, so that a readout without it shows
+    return out
+
+
+def capped_reference(ids, w, c):
+    """Whole sequence in float64; both layers share their tensors (the plan names one layer twice)."""
+    norm = lambda x, p: x / (x.abs().mean(-1, keepdim=True) + c.eps) * w[p]
+    d, hd = c.width, c.width // c.heads
+    x = w["tok"][ids] + w["pos"][:len(ids)]
+    for _ in range(2):
+        qkv = norm(x, "n1") @ w["qkv"].t()
+        q, k, v = (plain.split_heads(qkv[:, i * d:(i + 1) * d], c.heads) for i in range(3))
+        x = x + plain.merge_heads(plain.attention(q, k, v, hd ** -0.5)) @ w["out"].t()
+        x = x + plain.gelu_tanh(norm(x, "n2") @ w["up"].t() + w["up.b"]) @ w["down"].t() + w["down.b"]
+    return c.cap * torch.tanh((norm(x, "final") @ w["head"].t() + w["head.b"]) / c.cap)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_norm_and_a_readout_of_other_kinds(dtype, tmp_path):
+    register("norm", "toy_mean_abs_norm", MeanAbsNorm)
+    register("readout", "toy_capped_readout", CappedReadout)
+    bt.register_family(bt.Family("toy_capped", ("ToyCappedLM",), (), CappedConfig, capped_plan, capped_contract,
+                                 capped_init))
+    try:
+        config = CappedConfig()
+        stored = bt.write_random_model(str(tmp_path), config.to_dict(), seed=8)
+        model = bt.load_model(str(tmp_path), dtype=dtype)
+        engine = bt.Engine(model, max_tokens=512, graphs="always")
+        w = {k: v.double() for k, v in stored.items()}
+        gen = torch.Generator().manual_seed(2)
+        requests = [torch.randint(0, config.vocab_size, (n,), generator=gen).tolist() for n in (70, 9, 33)]
+        wants = [capped_reference(torch.tensor(r), w, config) for r in requests]
+        assert max(float(x.abs().max()) for x in wants) > 0.9 * config.cap          # the cap is at work
+        # bfloat16: the logits before the cap reach 10 and more and rounded weights move them by a per cent
+        # (measured: 0.05 to 0.08; a missing cap or another norm is off by 0.5 and more)
+        tol = 2e-5 if dtype == "float32" else 0.15
+        slots = [engine.open() for _ in requests]
+        cut = [len(r) - 6 for r in requests]
+        logits = engine.step([(s, r[:c]) for s, r, c in zip(slots, requests, cut)],
+                             want=[list(range(c)) for c in cut]).clone()
+        got, at = [[] for _ in requests], 0
+        for i, c in enumerate(cut):
+            got[i].append(logits[at:at + c])
+            at += c
+        for t in range(6):
+            logits = engine.step([(s, [r[c + t]]) for s, r, c in zip(slots, requests, cut)]).clone()
+            for i in range(len(requests)):
+                got[i].append(logits[i:i + 1])
+        assert engine.graph_replays >= 4
+        for i, want in enumerate(wants):
+            error = float((torch.cat(got[i]).cpu().double() - want).abs().max())
+            print(f"[toy norm and readout] {dtype} request {i}: max error {error:.3g}", flush=True)
+            assert error <= tol, f"request {i}"
+    finally:
+        unregister("norm", "toy_mean_abs_norm")
+        unregister("readout", "toy_capped_readout")
+        bt.unregister_family("toy_capped")

@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
                     [--repetitions 10] [--workload xl|small|medium|sweep] [--model xl|medium|small]
-                    [--kernel-batches 1,64] [--no-points] [--no-kernels] [--no-own]
+                    [--kernel-batches 1,64] [--sweep-part all|decode|prompts] [--no-points] [--no-kernels] [--no-own]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
 sequences, prefilled with 512 synthetic tokens each, is decoded towards 1,024.  A step is one

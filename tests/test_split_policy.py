@@ -61,6 +61,36 @@ def _runs(monkeypatch, n_seqs, context_limit, kv_heads=25, head_dim=64, bf16=Tru
     return attention.CausalSelfAttention.decode_runs(mixer, step, "cuda:0")
 
 
+def _prompt_runs(monkeypatch, capacity, n_seqs, context_limit, heads=25, head_dim=64, bf16=True, window=0, units=256):
+    from types import SimpleNamespace
+    from burn_transformers_amd.parts import attention
+    monkeypatch.setattr(attention, "compute_units", lambda device: units)
+    mixer = SimpleNamespace(heads=heads, head_dim=head_dim, window=window, plain_only=False)
+    step = SimpleNamespace(decode=False, context_limit=context_limit, dtype_is_bf16=bf16, n_seqs=n_seqs,
+                           token_capacity=capacity)
+    return attention.CausalSelfAttention.prompt_runs(mixer, step, "cuda:0")
+
+
+def test_prompt_runs_for_chunks_behind_long_contexts(monkeypatch):
+    """A chunk of a prompt has few tiles of 128 queries: their keys are cut into runs until the
+    work-groups fill the chip, each run at least 8 blocks of keys per 256 tokens of the step, none
+    while the class of context is 1,024 tokens or less, and only where the kernel that takes runs
+    is the one that runs (bfloat16, heads of 64, no window)."""
+    assert _prompt_runs(monkeypatch, 256, 1, 1024) == 1
+    assert _prompt_runs(monkeypatch, 256, 1, 2048) == 4            # 32 blocks in runs of 8
+    assert _prompt_runs(monkeypatch, 256, 1, 4096) == 5            # 2 tiles x 25 heads x 5 = 250 work-groups
+    assert _prompt_runs(monkeypatch, 256, 1, 8192) == 5
+    assert _prompt_runs(monkeypatch, 128, 1, 8192) == 8            # never more than eight
+    assert _prompt_runs(monkeypatch, 512, 2, 2048) == 2            # 5 tiles x 25 heads: two runs fit the chip, 16 blocks each
+    assert _prompt_runs(monkeypatch, 512, 2, 4096) == 2
+    assert _prompt_runs(monkeypatch, 1024, 1, 2048) == 1           # 8 blocks per 256 tokens: 32 a run here
+    assert _prompt_runs(monkeypatch, 2048, 1, 8192) == 1           # 16 tiles x 25 heads fill the chip already
+    assert _prompt_runs(monkeypatch, 256, 1, 8192, bf16=False) == 1
+    assert _prompt_runs(monkeypatch, 256, 1, 8192, head_dim=32) == 1
+    assert _prompt_runs(monkeypatch, 256, 1, 8192, window=512) == 1
+    assert _prompt_runs(monkeypatch, 256, 1, 8192, heads=4) == 8   # few heads: the runs are what fills the chip
+
+
 def test_decode_runs_at_measured_sizes(monkeypatch):
     # 25 heads of 64: bfloat16 is not cut at 1,024 keys, and best with 4 / 8 runs at 2,048 / 4,096
     assert _runs(monkeypatch, 1, 1024) == 1

@@ -661,8 +661,13 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
         elif deep_form_rows(m, k, a.stride(0), n, sliced=splits > 1):
             # short prompts and chunks: the tile kernel's deep forms (see ``deep_form_rows``)
             impl = "tile"
-            if variant == 0:     # tiles of 64 x 64 in four stages; of 128 x 64 beyond 128 rows where K is whole
-                variant = 5 if m <= 128 or splits > 1 else 7
+            if variant == 0:
+                # tiles of 64 x 64 in four stages, two work-groups to a compute unit.  (Tiles of 128 x
+                # 64 in three stages beyond 128 rows were the choice once: alone they measure the same
+                # at 256 rows, 19.9 against 19.5 us for 4800 x 1600, and lose at 129 to 192 rows, where
+                # the small tiles still have a compute unit each, 18.9 against 12.9 us; a prompt of 160
+                # tokens through 12 layers 1.08 -> 0.97 ms, of 256 tokens 1.20 -> 1.17 ms.)
+                variant = 5
         else:
             impl = "library" if splits == 1 and _library_takes(epilogue) and library_products() \
                 and _library_has_algorithm(a.stride(0), m, n, k, epilogue) else "tile"

@@ -658,7 +658,7 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
             impl = "skinny"
         elif dtype == FLOAT32:
             impl = "tile"
-        elif deep_form_rows(m, k, a.stride(0), n, sliced=splits > 1):
+        elif deep_form_rows(m, k, a.stride(0), n, sliced=splits > 1, scatters=epilogue.mode == EPI_QKV):
             # short prompts and chunks: the tile kernel's deep forms (see ``deep_form_rows``)
             impl = "tile"
             if variant == 0:
@@ -696,18 +696,23 @@ def gemm(a, w, epilogue, splits=1, impl="auto", variant=0, packed=None):
 
 
 DEEP_FORM_ROWS = 256          # most rows of a bfloat16 product that the tile kernel's deep forms take ...
-DEEP_FORM_SLICED_ROWS = 512   # ... and of one that leaves partial sums of slices of K pending
+DEEP_FORM_SLICED_ROWS = 512   # ... and of one that leaves partial sums of slices of K pending ...
+DEEP_FORM_SCATTER_ROWS = 384  # ... and of one that scatters keys and values into the cache
 
 
-def deep_form_rows(m, k, lda, n, sliced=False):
+def deep_form_rows(m, k, lda, n, sliced=False, scatters=False):
     """Whether a bfloat16 product of ``m`` rows is one for the tile kernel's deep forms (tiles of
     64 x 64 or 128 x 64 brought straight into LDS, several of them on their way at once): 65 to
     256 rows, where it has too few tiles of 128 x 128 to fill the chip and the vendor's library
     takes 16 to 24 us whatever the shape (measured at widths 1,600 and 6,400: these forms take a
     quarter to a third less); where the product may leave slices of K pending (``sliced``: the two
     products that add to the residual stream) up to 512 rows, and up to 45 % less.  Beyond, the
-    library wins.  The forms read K in tiles of 64 and address their operands with 32 bits."""
-    limit = DEEP_FORM_SLICED_ROWS if sliced else DEEP_FORM_ROWS
+    library wins.  The fused projection of a mixer (``scatters``) stays up to 384 rows: the
+    library's product cannot scatter keys and values into the cache, and the copy behind it costs
+    5 us (4800 x 1600 at 320 and 384 rows: 19.5 and 19.7 us here, 18.7 and 18.9 + 5.1 there; at 512
+    rows 28.4 against 20.8 + 5.0).  The forms read K in tiles of 64 and address their operands with
+    32 bits."""
+    limit = DEEP_FORM_SLICED_ROWS if sliced else DEEP_FORM_SCATTER_ROWS if scatters else DEEP_FORM_ROWS
     return 64 < m <= limit and k % 64 == 0 and m * lda * 2 < (1 << 32) and n * k * 2 < (1 << 32)
 
 
@@ -734,10 +739,10 @@ def deep_split_count(rows, columns, k, units=256):
     return max(1, min(4, splits, (k // 64) // 4))
 
 
-def prompt_products_in_library(m, n, k, lda):
+def prompt_products_in_library(m, n, k, lda, scatters=False):
     """Whether a bfloat16 product of a step of ``m`` rows goes to the vendor's library (which cannot
     scatter keys and values into the cache: the caller then copies them)."""
-    return m > 64 and not deep_form_rows(m, k, lda, n) and library_products() is not None
+    return m > 64 and not deep_form_rows(m, k, lda, n, scatters=scatters) and library_products() is not None
 
 
 def _library_has_algorithm(lda, m, n, k, epilogue):

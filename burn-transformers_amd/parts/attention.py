@@ -127,7 +127,8 @@ class CausalSelfAttention(Mixer):
         tokens = h.shape[0]
         kv = memory.kv()
         if memory.writes and step.dtype_is_bf16 and not self.plain_only and \
-                K.prompt_products_in_library(tokens, self.n_q + 2 * self.n_kv, self.width, h.stride(0) if hasattr(h, "stride") else self.width):
+                K.prompt_products_in_library(tokens, self.n_q + 2 * self.n_kv, self.width,
+                                             h.stride(0) if hasattr(h, "stride") else self.width, scatters=True):
             # a prompt: the vendor's library makes the whole projection, then keys and values are
             # copied into the cache; the queries are read where they lie
             qkv = step.buffer("attention.qkv", tokens, self.n_q + 2 * self.n_kv, step.dtype)

@@ -135,13 +135,15 @@ def test_whether_a_graph_pays_is_decided_by_the_median_of_the_measured_steps():
 
 def test_products_of_short_prompts_and_how_they_cut_k():
     """``deep_form_rows`` / ``deep_split_count``: 65 to 256 rows with K a multiple of 64 go to the
-    tile kernel's deep forms, up to 512 where slices of K may stay pending; a residual-writing one
+    tile kernel's deep forms, up to 512 where slices of K may stay pending and up to 384 where keys and
+    values are scattered into the cache (the vendor's library would need a copy behind it); a residual-writing one
     cuts K so that every work-group has a compute unit, or at most two share one, into at most four
     slices of at least four tiles of K."""
     from burn_transformers_amd.kernels.library import deep_form_rows, deep_split_count
     assert not deep_form_rows(64, 1600, 1600, 4800) and deep_form_rows(65, 1600, 1600, 4800)
     assert deep_form_rows(256, 1600, 1600, 4800) and not deep_form_rows(257, 1600, 1600, 4800)
     assert deep_form_rows(512, 1600, 1600, 1600, sliced=True) and not deep_form_rows(513, 1600, 1600, 1600, sliced=True)
+    assert deep_form_rows(384, 1600, 1600, 4800, scatters=True) and not deep_form_rows(385, 1600, 1600, 4800, scatters=True)
     assert not deep_form_rows(128, 1608, 1608, 4800)            # K in tiles of 64
     assert not deep_form_rows(128, 64, 1 << 25, 64)             # operands addressed with 32 bits
     assert deep_split_count(128, 1600, 1600) == 4 and deep_split_count(128, 1600, 6400) == 4
